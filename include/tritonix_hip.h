@@ -1,0 +1,120 @@
+/*
+ * tritonix_hip.h -- C ABI of libtritonix_hip.so, the gfx950 (MI355X) tiled-GEMM engine.
+ *
+ * Every entry point takes plain pointers and sizes; nothing here depends on
+ * PyTorch.  The library never allocates or frees device memory, never
+ * synchronises, and launches asynchronously on the stream the caller passes.
+ *
+ * Reference interfaces these entry points stand in for (paths are inside the
+ * ayghri/tritonix tree):
+ *   - the Triton launch `matmul_kernel[grid](a, b, c, m, n, k, 6 strides,
+ *     block_m=, block_n=, block_k=, group_m=, num_stages=, num_warps=)`
+ *     tritonix/ops/matmul.py:43-108, launched from :217-237;
+ *   - `gemm_splitk_kernel[grid](..., split_k=)` tritonix/ops/matmul.py:147-202,
+ *     launched from :240-264, with its `_zero_output` pre-run hook :205-210;
+ *   - `glu_kernel[grid](x, w12, z, m, n, k, 6 strides, block_*=, group_m=,
+ *     use_tf32=, activation=, num_stages=, num_warps=)`
+ *     tritonix/ops/swiglu.py:24-110 (phase 1 of swiglu_kernel :155-205);
+ *   - the int8 -> int32 kernel playground/test_int8_mma.py:7-42;
+ *   - `triton.OutOfResources` as raised by the Triton launcher and caught at
+ *     tritonix/autotune.py:134 (here: TNX_E_LDS + tnx_gemm_lds_bytes()).
+ */
+#ifndef TRITONIX_HIP_H
+#define TRITONIX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TNX_VERSION 1
+
+/* element types */
+enum tnx_dtype {
+  TNX_F16 = 0,  /* IEEE binary16 */
+  TNX_BF16 = 1, /* bfloat16 */
+  TNX_I8 = 2,   /* signed 8-bit */
+  TNX_I32 = 3,  /* signed 32-bit (output of the int8 path) */
+  TNX_F32 = 4   /* binary32 (output only) */
+};
+
+/* epilogues fused after the K loop (tritonix/ops/swiglu.py:98-104).
+ * For the GLU epilogues `n` is the interleaved width of B (even columns are
+ * the gate, odd columns the linear branch) and C has n/2 columns. */
+enum tnx_epilogue {
+  TNX_EPI_NONE = 0,
+  TNX_EPI_GLU_SILU = 1,     /* silu(gate) * lin   (activation == "silu")        */
+  TNX_EPI_GLU_SIGMOID = 2,  /* sigmoid(gate) * lin                               */
+  TNX_EPI_GLU_IDENTITY = 3  /* gate * lin (the reference's fall-through branch)  */
+};
+
+/* status codes */
+enum tnx_status {
+  TNX_OK = 0,
+  TNX_E_INVALID = 1,     /* null pointer, negative size, bad enum                     */
+  TNX_E_UNSUPPORTED = 2, /* no kernel is built for this tile / dtype / layout combo   */
+  TNX_E_LDS = 3,         /* the tile config needs more LDS than one CU has            */
+  TNX_E_WORKSPACE = 4,   /* split_k > 1 and the workspace is missing or too small     */
+  TNX_E_HIP = 5          /* the HIP runtime reported an error (see tnx_last_hip_error) */
+};
+
+/* Per-CU LDS capacity on gfx950; the budget tile configs are pruned against. */
+#define TNX_LDS_LIMIT_BYTES 163840
+
+typedef struct tnx_gemm_args {
+  const void* a;   /* [m, k], element strides stride_am / stride_ak             */
+  const void* b;   /* [k, n], element strides stride_bk / stride_bn             */
+  void* c;         /* [m, n] (or [m, n/2] with a GLU epilogue)                  */
+  int64_t m, n, k;
+  int64_t stride_am, stride_ak;
+  int64_t stride_bk, stride_bn;
+  int64_t stride_cm, stride_cn;
+  int32_t in_dtype;   /* tnx_dtype of a and b                                    */
+  int32_t out_dtype;  /* tnx_dtype of c                                          */
+  int32_t block_m, block_n, block_k; /* workgroup tile                           */
+  int32_t group_m;    /* rows of tiles per L2 super-group (tl.swizzle2d size_g)  */
+  int32_t split_k;    /* 1 = no split; >1 = K is cut into split_k slices         */
+  int32_t num_stages; /* LDS ring depth of the global->LDS pipeline              */
+  int32_t num_warps;  /* wavefronts (64 lanes) per workgroup: 4 or 8             */
+  int32_t epilogue;   /* tnx_epilogue                                            */
+  void* workspace;    /* device scratch for split_k > 1, else may be NULL        */
+  size_t workspace_bytes;
+  void* stream;       /* hipStream_t; NULL = the null stream                     */
+} tnx_gemm_args;
+
+/* Launch one GEMM.  Returns a tnx_status.  Asynchronous. */
+int tnx_gemm(const tnx_gemm_args* args);
+
+/* Bytes of device scratch tnx_gemm needs for these args (0 when split_k <= 1).
+ * The contents need no initialisation: the kernels own it (this replaces the
+ * reference's `_zero_output` hook, tritonix/ops/matmul.py:205-210). */
+size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* args);
+
+/* LDS bytes per workgroup the tile config in `args` would use.  Pure host
+ * arithmetic, no GPU needed: lets the tuner's trie prune a config without
+ * launching it.  Returns -1 if the config is malformed. */
+int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* args);
+
+/* TNX_OK if tnx_gemm would accept these args (pointers are not inspected),
+ * otherwise the status it would return.  Pure host arithmetic. */
+int tnx_gemm_supported(const tnx_gemm_args* args);
+
+/* Fill block_m/n/k, group_m, split_k, num_stages, num_warps of `args` with a
+ * built-in choice for its shape and dtype (used when nothing was tuned). */
+int tnx_gemm_default_config(tnx_gemm_args* args);
+
+/* Number of compiled tile kernels, and a description of the i-th one:
+ * "dtype bm bn bk warps stages" as a NUL-terminated string (static storage). */
+int tnx_kernel_count(void);
+const char* tnx_kernel_name(int i);
+
+const char* tnx_strerror(int status);
+int tnx_last_hip_error(void); /* hipError_t of the last TNX_E_HIP on this thread */
+int tnx_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITONIX_HIP_H */

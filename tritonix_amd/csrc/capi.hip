@@ -1,0 +1,214 @@
+// C ABI of libtritonix_hip.so: argument checking, tile-kernel lookup, launch.
+// Declarations and the reference interfaces they replace: include/tritonix_hip.h
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/tritonix_hip.h"
+#include "registry.h"
+
+using namespace tnx;
+
+extern "C" const KernelGroup* tnx_kernel_groups(int* ngroups);  // generated
+
+static thread_local int g_last_hip_error = 0;
+
+static int elem_size(int dt) { return dt == TNX_I8 ? 1 : (dt == TNX_F16 || dt == TNX_BF16) ? 2 : 4; }
+
+static const KernelEntry* find_entry(const tnx_gemm_args* a) {
+  int ng = 0;
+  const KernelGroup* g = tnx_kernel_groups(&ng);
+  for (int i = 0; i < ng; ++i)
+    for (int j = 0; j < g[i].count; ++j) {
+      const KernelEntry& e = g[i].entries[j];
+      if (e.dtype == a->in_dtype && e.bm == a->block_m && e.bn == a->block_n && e.bk == a->block_k &&
+          e.nw == a->num_warps && e.stages == a->num_stages)
+        return &e;
+    }
+  return nullptr;
+}
+
+static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+// LDS bytes of a tile config, whether or not a kernel is built for it
+static int64_t lds_bytes_of(const tnx_gemm_args* a) {
+  if (a->block_m <= 0 || a->block_n <= 0 || a->block_k <= 0 || a->num_stages <= 0) return -1;
+  int es = elem_size(a->in_dtype);
+  return (int64_t)a->num_stages * ((int64_t)a->block_m * a->block_k + (int64_t)a->block_k * a->block_n) * es;
+}
+
+static int check_common(const tnx_gemm_args* a) {
+  if (!a) return TNX_E_INVALID;
+  if (a->m < 0 || a->n < 0 || a->k < 0) return TNX_E_INVALID;
+  if (a->in_dtype != TNX_F16 && a->in_dtype != TNX_BF16 && a->in_dtype != TNX_I8) return TNX_E_INVALID;
+  if (a->epilogue < TNX_EPI_NONE || a->epilogue > TNX_EPI_GLU_IDENTITY) return TNX_E_INVALID;
+  if (a->block_m <= 0 || a->block_n <= 0 || a->block_k <= 0 || a->group_m <= 0 || a->split_k <= 0 ||
+      a->num_stages <= 0 || a->num_warps <= 0)
+    return TNX_E_INVALID;
+  // output type is tied to the input type: f16->f16, bf16->bf16, i8->i32
+  int want_out = a->in_dtype == TNX_I8 ? TNX_I32 : a->in_dtype;
+  if (a->out_dtype != want_out) return TNX_E_UNSUPPORTED;
+  if (a->epilogue != TNX_EPI_NONE && (a->in_dtype == TNX_I8 || (a->n & 1))) return TNX_E_UNSUPPORTED;
+  if (a->m > 0x7fffffff || a->n > 0x7fffffff || a->k > 0x7fffffff) return TNX_E_UNSUPPORTED;
+  return TNX_OK;
+}
+
+static bool fast_layout(const tnx_gemm_args* a) {
+  const int es = elem_size(a->in_dtype);
+  const int vec = 16 / es;
+  if (a->stride_ak != 1 || a->stride_bn != 1) return false;
+  if (a->k % a->block_k != 0 || a->k == 0) return false;
+  if ((a->stride_am * es) % 16 != 0 || (a->stride_bk * es) % 16 != 0) return false;
+  if (a->stride_am < 0 || a->stride_bk < 0) return false;
+  if (((uintptr_t)a->a & 15) || ((uintptr_t)a->b & 15)) return false;
+  if (a->n % vec != 0 || a->n < vec) return false;
+  // per-lane DMA offsets are 32-bit
+  if ((int64_t)a->block_m * a->stride_am * es >= (1ll << 32)) return false;
+  if ((int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es >= (1ll << 32)) return false;
+  return true;
+}
+
+extern "C" int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* a) {
+  if (!a) return -1;
+  return lds_bytes_of(a);
+}
+
+extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
+  if (!a || a->split_k <= 1 || a->m <= 0 || a->n <= 0) return 0;
+  return (size_t)a->split_k * (size_t)a->m * (size_t)a->n * 4;
+}
+
+static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs) {
+  int st = check_common(a);
+  if (st != TNX_OK) return st;
+  int64_t lds = lds_bytes_of(a);
+  if (lds > TNX_LDS_LIMIT_BYTES) return TNX_E_LDS;
+  const KernelEntry* e = find_entry(a);
+  if (!e) return TNX_E_UNSUPPORTED;
+  tnx_gemm_args tmp = *a;
+  if (!inspect_ptrs) { tmp.a = nullptr; tmp.b = nullptr; }
+  bool f = fast_layout(&tmp);
+  if (!f && !e->generic) return TNX_E_UNSUPPORTED;
+  int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
+  if (tiles * a->split_k > 0x7fffffffll) return TNX_E_UNSUPPORTED;
+  if (out) *out = e;
+  if (fast) *fast = f;
+  return TNX_OK;
+}
+
+extern "C" int tnx_gemm_supported(const tnx_gemm_args* a) { return supported_impl(a, nullptr, nullptr, false); }
+
+extern "C" int tnx_gemm(const tnx_gemm_args* a) {
+  const KernelEntry* e = nullptr;
+  bool fast = false;
+  int st = supported_impl(a, &e, &fast, true);
+  if (st != TNX_OK) return st;
+  if (!a->a || !a->b || !a->c) {
+    if (a->m == 0 || a->n == 0) return TNX_OK;
+    if (!a->c || (a->k > 0 && (!a->a || !a->b))) return TNX_E_INVALID;
+  }
+  if (a->m == 0 || a->n == 0) return TNX_OK;
+  if (a->split_k > 1 && (!a->workspace || a->workspace_bytes < tnx_gemm_workspace_bytes(a))) return TNX_E_WORKSPACE;
+
+  const int es_out = elem_size(a->out_dtype);
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t*)a->a;
+  p.b = (const uint8_t*)a->b;
+  p.c = (uint8_t*)a->c;
+  p.ws = (uint8_t*)a->workspace;
+  p.m = a->m; p.n = a->n; p.k = a->k;
+  p.sam = a->stride_am; p.sak = a->stride_ak;
+  p.sbk = a->stride_bk; p.sbn = a->stride_bn;
+  p.scm = a->stride_cm; p.scn = a->stride_cn;
+  p.tiles_m = (int)((a->m + a->block_m - 1) / a->block_m);
+  p.tiles_n = (int)((a->n + a->block_n - 1) / a->block_n);
+  p.group_m = a->group_m;
+  p.split_k = a->split_k;
+  int kt_total = (int)((a->k + a->block_k - 1) / a->block_k);
+  p.ktiles_per_split = (kt_total + a->split_k - 1) / a->split_k;
+  p.epilogue = a->epilogue;
+  p.out_dtype = a->out_dtype;
+  p.c_vec_ok = a->stride_cn == 1 && (a->stride_cm % 4) == 0 && (((uintptr_t)a->c) % (4 * es_out)) == 0;
+
+  hipStream_t stream = (hipStream_t)a->stream;
+  unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * a->split_k);
+  hipError_t err = (fast ? e->fast : e->generic)(p, grid, stream);
+  if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+
+  if (a->split_k > 1) {
+    int64_t ncols = a->epilogue == TNX_EPI_NONE ? a->n : a->n / 2;
+    int64_t total = a->m * ncols;
+    unsigned rgrid = (unsigned)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    if (a->in_dtype == TNX_I8)
+      hipLaunchKernelGGL((splitk_reduce_kernel<int>), dim3(rgrid), dim3(256), 0, stream, (const int*)p.ws, p.c, p.m, p.n,
+                         p.scm, p.scn, p.split_k, p.epilogue, p.out_dtype);
+    else
+      hipLaunchKernelGGL((splitk_reduce_kernel<float>), dim3(rgrid), dim3(256), 0, stream, (const float*)p.ws, p.c, p.m,
+                         p.n, p.scm, p.scn, p.split_k, p.epilogue, p.out_dtype);
+    err = hipGetLastError();
+    if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+  }
+  return TNX_OK;
+}
+
+extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
+  if (!a) return TNX_E_INVALID;
+  const int es = elem_size(a->in_dtype);
+  a->group_m = 8;
+  a->split_k = 1;
+  a->num_warps = 4;
+  if (a->m <= 64) {
+    // skinny: stream B, split K to fill the chip
+    a->block_m = 64; a->block_n = 128; a->block_k = 64 / es * 2 > 64 ? 128 : 64; a->num_stages = 3;
+    a->block_k = es == 1 ? 128 : 64;
+    int64_t tiles = (a->n + a->block_n - 1) / a->block_n;
+    int64_t kt = (a->k + a->block_k - 1) / a->block_k;
+    int s = 1;
+    while (tiles * s < 512 && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
+    a->split_k = s;
+  } else if (a->m >= 2048 && a->n >= 2048) {
+    a->block_m = 256; a->block_n = 256; a->block_k = es == 1 ? 128 : 64; a->num_stages = 2;
+  } else {
+    a->block_m = 128; a->block_n = 128; a->block_k = es == 1 ? 128 : 64; a->num_stages = 3;
+  }
+  return TNX_OK;
+}
+
+extern "C" int tnx_kernel_count(void) {
+  int ng = 0, n = 0;
+  const KernelGroup* g = tnx_kernel_groups(&ng);
+  for (int i = 0; i < ng; ++i) n += g[i].count;
+  return n;
+}
+
+extern "C" const char* tnx_kernel_name(int idx) {
+  static thread_local char buf[96];
+  int ng = 0;
+  const KernelGroup* g = tnx_kernel_groups(&ng);
+  for (int i = 0; i < ng; ++i) {
+    if (idx < g[i].count) {
+      const KernelEntry& e = g[i].entries[idx];
+      const char* dn = e.dtype == TNX_F16 ? "f16" : e.dtype == TNX_BF16 ? "bf16" : "i8";
+      snprintf(buf, sizeof(buf), "%s %d %d %d %d %d%s", dn, e.bm, e.bn, e.bk, e.nw, e.stages, e.generic ? " generic" : "");
+      return buf;
+    }
+    idx -= g[i].count;
+  }
+  return nullptr;
+}
+
+extern "C" const char* tnx_strerror(int status) {
+  switch (status) {
+    case TNX_OK: return "ok";
+    case TNX_E_INVALID: return "invalid argument";
+    case TNX_E_UNSUPPORTED: return "no kernel is built for this tile / dtype / layout";
+    case TNX_E_LDS: return "tile configuration exceeds the per-CU LDS budget";
+    case TNX_E_WORKSPACE: return "split-K workspace missing or too small";
+    case TNX_E_HIP: return "HIP runtime error";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int tnx_last_hip_error(void) { return g_last_hip_error; }
+extern "C" int tnx_version(void) { return TNX_VERSION; }

@@ -1,0 +1,619 @@
+// Tiled GEMM for gfx950 (MI355X): C[m,n] = A[m,k] @ B[k,n], optional split-K
+// partials and a fused GLU epilogue.
+//
+// What it computes follows tritonix/ops/matmul.py:43-108 (matmul_kernel),
+// :147-202 (gemm_splitk_kernel) and tritonix/ops/swiglu.py:24-110 (glu_kernel):
+// a block_m x block_n output tile per workgroup, a K loop of block_k slabs with
+// fp32 (int32 for int8) accumulation, an M/N-masked store.  How it computes it
+// is specific to CDNA4:
+//   * global -> LDS with the 16-byte direct-to-LDS load (no VGPR staging), a
+//     ring of STAGES LDS slabs, one workgroup barrier per K slab;
+//   * A fragments with ds_read_b128, B fragments (B is row-major [k,n], MFMA
+//     wants k-contiguous lanes) with the transposing ds_read_b64_tr_b16/_b8;
+//   * XOR-swizzled 16-byte chunks so neither the DMA writes nor the fragment
+//     reads collide on LDS banks;
+//   * v_mfma_f32_32x32x16 (bf16/f16), v_mfma_i32_32x32x32_i8, or the 16x16
+//     shapes when a wave's tile is narrower than 32;
+//   * a 1-D grid whose block index is remapped XCD-first, then by the
+//     group-M order of tl.swizzle2d (tritonix/ops/matmul.py:70).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tnx {
+
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+#define TNX_LDS(T, addr) ((T __attribute__((address_space(3)))*)(uintptr_t)(addr))
+
+enum { DT_F16 = 0, DT_BF16 = 1, DT_I8 = 2, DT_I32 = 3, DT_F32 = 4 };
+enum { EPI_NONE = 0, EPI_GLU_SILU = 1, EPI_GLU_SIGMOID = 2, EPI_GLU_IDENTITY = 3 };
+
+struct GemmParams {
+  const uint8_t* a;
+  const uint8_t* b;
+  uint8_t* c;
+  uint8_t* ws;            // split-K partials [split][m][n], fp32 or int32
+  int64_t m, n, k;
+  int64_t sam, sak;       // element strides of A
+  int64_t sbk, sbn;       // element strides of B
+  int64_t scm, scn;       // element strides of C
+  int tiles_m, tiles_n;
+  int group_m;
+  int split_k;
+  int ktiles_per_split;   // K slabs handled by one split
+  int epilogue;
+  int out_dtype;
+  bool c_vec_ok;          // C allows 4-element vector stores along n (stride_cn == 1, aligned)
+};
+
+// ---------------------------------------------------------------------------
+// element tags
+// ---------------------------------------------------------------------------
+struct TagF16 { static constexpr int ES = 2; static constexpr int ID = DT_F16; typedef float acc_s; };
+struct TagBF16 { static constexpr int ES = 2; static constexpr int ID = DT_BF16; typedef float acc_s; };
+struct TagI8 { static constexpr int ES = 1; static constexpr int ID = DT_I8; typedef int acc_s; };
+
+template <class T, int MI> struct Mma;
+template <> struct Mma<TagBF16, 32> {
+  typedef f32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<TagBF16, 16> {
+  typedef f32x4 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<TagF16, 32> {
+  typedef f32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<TagF16, 16> {
+  typedef f32x4 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<TagI8, 32> {
+  typedef i32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<TagI8, 16> {
+  typedef i32x4 acc_t;
+  static __device__ __forceinline__ acc_t run(i32x4 a, i32x4 b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// tile-id remap.  Workgroups are dealt round-robin to the 8 XCDs (each has its
+// own L2), so consecutive *logical* tile ids are first gathered per XCD, then
+// ordered group-M-first exactly like tl.swizzle2d on the row-major tile index
+// (triton/language/standard.py:80-116, called at tritonix/ops/matmul.py:70).
+// ---------------------------------------------------------------------------
+__host__ __device__ inline int xcd_remap(int pid, int total, int nxcd) {
+  int q = total / nxcd, r = total % nxcd;
+  int x = pid % nxcd, idx = pid / nxcd;
+  int start = x * q + (x < r ? x : r);
+  return start + idx;
+}
+
+__host__ __device__ inline void swizzle2d(int i, int j, int size_i, int size_j, int size_g, int* oi, int* oj) {
+  int ij = i * size_j + j;
+  int size_gj = size_g * size_j;
+  int group_id = ij / size_gj;
+  int off_i = group_id * size_g;
+  int g = size_i - off_i < size_g ? size_i - off_i : size_g;
+  int r = ij % size_gj;
+  *oi = off_i + r % g;
+  *oj = r / g;
+}
+
+// vmcnt-only wait (lgkmcnt and expcnt left at "no wait") in the gfx9 encoding
+#define TNX_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | ((((n) >> 4) & 0x3) << 14) | 0x0F70)
+
+// 16 bytes per lane, global -> LDS without touching VGPRs.  LDS destination is
+// lds_base + lane*16 (lds_base wave-uniform, carried in M0).
+__device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base), "v"(voff), "s"(sbase)
+               : "memory");
+}
+
+template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
+template <> __device__ __forceinline__ i32x2 lds_read_tr<2>(uint32_t addr) {
+  return __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(TNX_LDS(i16x4, addr)));
+}
+template <> __device__ __forceinline__ i32x2 lds_read_tr<1>(uint32_t addr) {
+  return __builtin_amdgcn_ds_read_tr8_b64_v2i32(TNX_LDS(i32x2, addr));
+}
+
+__device__ __forceinline__ float quad_swap1(float v) {
+  // lanes (0,1,2,3) <- (1,0,3,2)
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float glu_gate(float g, int epi) {
+  if (epi == EPI_GLU_IDENTITY) return g;
+  float s = 1.0f / (1.0f + __expf(-g));
+  return epi == EPI_GLU_SILU ? g * s : s;
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                             // round to nearest even
+  return (uint16_t)(u >> 16);
+}
+
+template <class ACC> __device__ __forceinline__ void store_out(uint8_t* c, int64_t off, ACC v, int out_dtype);
+template <> __device__ __forceinline__ void store_out<float>(uint8_t* c, int64_t off, float v, int out_dtype) {
+  if (out_dtype == DT_BF16) ((uint16_t*)c)[off] = f32_to_bf16(v);
+  else if (out_dtype == DT_F16) ((_Float16*)c)[off] = (_Float16)v;
+  else ((float*)c)[off] = v;
+}
+template <> __device__ __forceinline__ void store_out<int>(uint8_t* c, int64_t off, int v, int out_dtype) {
+  ((int*)c)[off] = v;
+}
+
+// ---------------------------------------------------------------------------
+// static description of one tile configuration
+// ---------------------------------------------------------------------------
+template <class T, int BM_, int BN_, int BK_, int NW_, int STAGES_>
+struct TileCfg {
+  static constexpr int ES = T::ES;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, NW = NW_, STAGES = STAGES_;
+  static constexpr int THREADS = NW * 64;
+  static constexpr int WGM = (NW == 4) ? 2 : (BM > BN ? 4 : 2);  // wave grid
+  static constexpr int WGN = NW / WGM;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;            // wave tile
+  static constexpr int MI = (WTM % 32 == 0 && WTN % 32 == 0) ? 32 : 16;
+  static constexpr int TM = WTM / MI, TN = WTN / MI;
+  static constexpr int KB = (MI == 32) ? 32 : 64;                 // k bytes one MFMA consumes
+  static constexpr int MMA_K = KB / ES;
+  static constexpr int KSTEPS = (BK * ES) / KB;
+  static constexpr int KGROUPS = 64 / MI;                         // lane groups along k
+  static constexpr int ROWB_A = BK * ES, CPR_A = ROWB_A / 16;
+  static constexpr int ROWB_B = BN * ES, CPR_B = ROWB_B / 16;
+  static constexpr int A_BYTES = BM * ROWB_A, B_BYTES = BK * ROWB_B;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int A_LOADS = A_BYTES / 1024, B_LOADS = B_BYTES / 1024;  // wave-wide 1 KiB DMA ops
+  static constexpr int A_LPW = (A_LOADS + NW - 1) / NW, B_LPW = (B_LOADS + NW - 1) / NW;
+  static constexpr int LPW = A_LPW + B_LPW;                       // DMA ops one wave issues per slab
+  static constexpr int ACC_N = (MI == 32) ? 16 : 4;
+  static constexpr bool VALID =
+      (WTM % 16 == 0) && (WTN % 16 == 0) && (BK * ES) % KB == 0 && KSTEPS >= 1 && CPR_A >= 4 &&
+      (ES == 2 ? CPR_B >= 8 : CPR_B >= 8) && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
+      LDS_BYTES <= 163840 && TM * TN * ACC_N <= 256 && (STAGES - 2) * LPW <= 63 && STAGES >= 2;
+
+  // chunk-index XOR applied to row `row` of the A slab
+  static __host__ __device__ constexpr int swzA(int row) {
+    return CPR_A >= 8 ? ((row & 7) ^ ((row >> 3) & 1)) : (((row >> 1) & 3) ^ ((row >> 3) & 1));
+  }
+  // chunk-index XOR applied to row `row` (a k index) of the B slab
+  static __host__ __device__ constexpr int swzB(int row) {
+    if (ES == 2) {
+      if (CPR_B >= 16) { int k = row & 3; return (2 * k + (k >> 1)) << 1; }
+      return (row & 3) << 1;
+    } else {
+      if (CPR_B >= 16) { int k = row & 7; return 2 * k + (k >> 2); }
+      return row & 7;
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// output conversion and the store of one accumulator tile set
+// ---------------------------------------------------------------------------
+struct OutBF16 { typedef uint16_t raw; static __device__ __forceinline__ raw cvt(float v) { return f32_to_bf16(v); } };
+struct OutF16 {
+  typedef uint16_t raw;
+  static __device__ __forceinline__ raw cvt(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <class T> struct OutOf;
+template <> struct OutOf<TagBF16> { typedef OutBF16 type; };
+template <> struct OutOf<TagF16> { typedef OutF16 type; };
+template <> struct OutOf<TagI8> { typedef int type; };
+
+template <class O, class S> struct Cvt { typedef typename O::raw raw; static __device__ __forceinline__ raw run(S v) { return O::cvt((float)v); } };
+template <> struct Cvt<float, float> { typedef float raw; static __device__ __forceinline__ float run(float v) { return v; } };
+template <> struct Cvt<int, int> { typedef int raw; static __device__ __forceinline__ int run(int v) { return v; } };
+
+// GLU != 0: columns (2c, 2c+1) hold (gate, linear); output column c.
+template <class T, class C, class O, int GLU, class ACC>
+__device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, int64_t gm_base, int64_t gn_base,
+                                               int64_t m, int64_t n, int64_t scm, int64_t scn, bool vec_ok, int epi) {
+  typedef typename T::acc_s acc_s;
+  typedef Cvt<O, acc_s> CV;
+  typedef typename CV::raw raw;
+  constexpr int MI = C::MI;
+  constexpr int NGRP = C::ACC_N / 4;        // groups of four consecutive columns per accumulator tile
+  raw* cp = (raw*)cbase;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+    const int64_t gm = gm_base + i * MI;
+    if (gm >= m) continue;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < NGRP; ++g) {
+        const int64_t gn = gn_base + j * MI + g * 8;
+        acc_s v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+        if (GLU) {
+          const int64_t nh = n >> 1, gc = gn >> 1;
+          raw z0 = CV::run((acc_s)(glu_gate((float)v0, epi) * (float)v1));
+          raw z1 = CV::run((acc_s)(glu_gate((float)v2, epi) * (float)v3));
+          raw* dst = cp + gm * scm + gc * scn;
+          if (vec_ok && gc + 1 < nh) {
+            if constexpr (sizeof(raw) == 2) *(uint32_t*)dst = (uint32_t)z0 | ((uint32_t)z1 << 16);
+            else { dst[0] = z0; dst[1] = z1; }
+          } else {
+            if (gc < nh) dst[0] = z0;
+            if (gc + 1 < nh) dst[scn] = z1;
+          }
+        } else {
+          raw r0 = CV::run(v0), r1 = CV::run(v1), r2 = CV::run(v2), r3 = CV::run(v3);
+          raw* dst = cp + gm * scm + gn * scn;
+          if (vec_ok && gn + 3 < n) {
+            if constexpr (sizeof(raw) == 2) {
+              uint2 pk;
+              pk.x = (uint32_t)r0 | ((uint32_t)r1 << 16);
+              pk.y = (uint32_t)r2 | ((uint32_t)r3 << 16);
+              *(uint2*)dst = pk;
+            } else {
+              uint4 pk;
+              pk.x = __builtin_bit_cast(uint32_t, r0); pk.y = __builtin_bit_cast(uint32_t, r1);
+              pk.z = __builtin_bit_cast(uint32_t, r2); pk.w = __builtin_bit_cast(uint32_t, r3);
+              *(uint4*)dst = pk;
+            }
+          } else {
+            if (gn < n) dst[0] = r0;
+            if (gn + 1 < n) dst[scn] = r1;
+            if (gn + 2 < n) dst[2 * scn] = r2;
+            if (gn + 3 < n) dst[3 * scn] = r3;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// the kernel
+// ---------------------------------------------------------------------------
+template <class T, class C, bool FAST>
+__global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
+  constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
+  constexpr int MI = C::MI, TM = C::TM, TN = C::TN;
+  typedef Mma<T, MI> MMA;
+  typedef typename MMA::acc_t acc_t;
+  typedef typename T::acc_s acc_s;
+
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[C::LDS_BYTES];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- which tile / split ------------------------------------------------
+  const int ntiles = p.tiles_m * p.tiles_n;
+  int bid = blockIdx.x;
+  const int split = bid / ntiles;
+  bid -= split * ntiles;
+  const int logical = xcd_remap(bid, ntiles, 8);
+  int pid_m, pid_n;
+  swizzle2d(logical / p.tiles_n, logical % p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, &pid_m, &pid_n);
+  const int64_t m0 = (int64_t)pid_m * BM, n0 = (int64_t)pid_n * BN;
+
+  const int kt_total = (int)((p.k + BK - 1) / BK);
+  const int kt0 = split * p.ktiles_per_split;
+  int kt1 = kt0 + p.ktiles_per_split;
+  if (kt1 > kt_total) kt1 = kt_total;
+  const int KT = kt1 > kt0 ? kt1 - kt0 : 0;          // slabs of this workgroup
+  // FAST kernels are only launched when k % BK == 0 and A, B are row-major
+  // and 16-byte aligned: every slab goes through the DMA path.  Otherwise every
+  // slab goes through the element-wise loader.
+  const int kt_dma = FAST ? KT : 0;
+
+  // ---- DMA addressing (FAST): per-lane byte offsets, constant over the K loop
+  uint32_t a_voff[C::A_LPW], b_voff[C::B_LPW];
+  const uint8_t* a_sbase = p.a;
+  const uint8_t* b_sbase = p.b;
+  if (FAST) {
+    const int64_t lda = p.sam, ldb = p.sbk;
+    a_sbase = p.a + (m0 * lda + (int64_t)kt0 * BK) * ES;
+    b_sbase = p.b + ((int64_t)kt0 * BK * ldb + n0) * ES;
+    const int64_t mrem = p.m - 1 - m0;  // last valid row inside this tile
+#pragma unroll
+    for (int q = 0; q < C::A_LPW; ++q) {
+      int P = (q * NW + wave) * 64 + lane;
+      int row = P / C::CPR_A, cs = P % C::CPR_A;
+      int c = cs ^ C::swzA(row);
+      int64_t r = row < mrem ? row : mrem;
+      a_voff[q] = (uint32_t)(r * lda * ES + c * 16);
+    }
+#pragma unroll
+    for (int q = 0; q < C::B_LPW; ++q) {
+      int P = (q * NW + wave) * 64 + lane;
+      int row = P / C::CPR_B, cs = P % C::CPR_B;
+      int c = cs ^ C::swzB(row);
+      if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
+      b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
+    }
+  }
+
+  // element-wise loader: any strides, any ragged edge, zero fill.  Used for
+  // the K-tail slab of FAST kernels and for every slab otherwise.
+  auto load_slab_generic = [&](int kt_global, uint32_t stage_base) {
+    const int64_t k0 = (int64_t)kt_global * BK;
+    for (int idx = tid; idx < BM * BK; idx += C::THREADS) {
+      int row = idx / BK, kk = idx % BK;
+      int64_t gm = m0 + row, gk = k0 + kk;
+      uint32_t dst = stage_base + row * C::ROWB_A + ((((kk * ES) >> 4) ^ C::swzA(row)) << 4) + ((kk * ES) & 15);
+      if (ES == 2) {
+        uint16_t v = 0;
+        if (gm < p.m && gk < p.k) v = ((const uint16_t*)p.a)[gm * p.sam + gk * p.sak];
+        *TNX_LDS(uint16_t, dst) = v;
+      } else {
+        uint8_t v = 0;
+        if (gm < p.m && gk < p.k) v = p.a[gm * p.sam + gk * p.sak];
+        *TNX_LDS(uint8_t, dst) = v;
+      }
+    }
+    for (int idx = tid; idx < BK * BN; idx += C::THREADS) {
+      int row = idx / BN, nn = idx % BN;
+      int64_t gk = k0 + row, gn = n0 + nn;
+      uint32_t dst = stage_base + C::A_BYTES + row * C::ROWB_B + ((((nn * ES) >> 4) ^ C::swzB(row)) << 4) + ((nn * ES) & 15);
+      if (ES == 2) {
+        uint16_t v = 0;
+        if (gk < p.k && gn < p.n) v = ((const uint16_t*)p.b)[gk * p.sbk + gn * p.sbn];
+        *TNX_LDS(uint16_t, dst) = v;
+      } else {
+        uint8_t v = 0;
+        if (gk < p.k && gn < p.n) v = p.b[gk * p.sbk + gn * p.sbn];
+        *TNX_LDS(uint8_t, dst) = v;
+      }
+    }
+  };
+
+  // one DMA op (q-th of this wave) of local slab t, into ring slot t % STAGES
+  auto dma_op = [&](int q, uint32_t stage_base) {
+    if (q < C::A_LPW) {
+      dma16(a_sbase, a_voff[q], stage_base + (q * NW + wave) * 1024);
+    } else {
+      dma16(b_sbase, b_voff[q - C::A_LPW], stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
+    }
+  };
+  auto dma_advance = [&]() {
+    a_sbase += BK * ES;
+    b_sbase += (int64_t)BK * p.sbk * ES;
+  };
+  auto stage_of = [&](int t) { return lds0 + (uint32_t)(t % STAGES) * C::STAGE_BYTES; };
+
+  // ---- fragment addressing ----------------------------------------------
+  const int wy = wave / C::WGN, wx = wave % C::WGN;
+  const int a_row = wy * C::WTM + (lane % MI);
+  const int a_kg = lane / MI;
+  const int a_sw = C::swzA(a_row);
+  uint32_t a_koff[C::KSTEPS];   // byte offset inside the A slab, per k step
+#pragma unroll
+  for (int ks = 0; ks < C::KSTEPS; ++ks)
+    a_koff[ks] = a_row * C::ROWB_A + (((ks * (C::KB / 16) + a_kg) ^ a_sw) << 4);
+
+  const int blk = lane >> 4, li = lane & 15;
+  const int b_kg = (MI == 32) ? (blk >> 1) : blk;
+  const int b_sub = (ES == 2) ? (li >> 2) : (li >> 1);               // k row inside the transposed block
+  const int b_colb0 = (wx * C::WTN + ((MI == 32) ? 16 * (blk & 1) : 0)) * ES + ((ES == 2) ? 8 * (li & 3) : 8 * (li & 1));
+  constexpr int RPR = 8 / ES;                                       // k rows one transposing read covers
+  const int b_sw = C::swzB(b_sub);
+  uint32_t b_joff[TN];          // byte offset inside the B slab, per column block
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int colb = b_colb0 + j * MI * ES;
+    b_joff[j] = (uint32_t)(((16 / ES) * b_kg + b_sub) * C::ROWB_B) + (((colb >> 4) ^ b_sw) << 4) + (colb & 15);
+  }
+
+  acc_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{};
+
+  // two register sets of fragments: one being multiplied, one being filled
+  i32x4 fa[2][TM];
+  i32x2 fb[2][TN][2];
+  constexpr int NREAD = 2 * TN + TM, NMMA = TM * TN;
+  constexpr int RPM = (NREAD + NMMA - 1) / NMMA;        // LDS reads slotted behind each MFMA
+  constexpr int DPM = (C::LPW + NMMA - 1) / NMMA;       // DMA ops slotted behind each MFMA
+
+  auto read_one = [&](int set, int idx, uint32_t sa, uint32_t sb, int ks) {
+    if (idx < 2 * TN) {
+      int j = idx >> 1, h = idx & 1;
+      fb[set][j][h] = lds_read_tr<ES>(sb + b_joff[j] + ks * C::MMA_K * C::ROWB_B + h * RPR * C::ROWB_B);
+    } else {
+      int i = idx - 2 * TN;
+      fa[set][i] = *TNX_LDS(i32x4, sa + a_koff[ks] + i * MI * C::ROWB_A);
+    }
+  };
+  auto mma_one = [&](int set, int idx) {
+    int i = idx / TN, j = idx % TN;
+    i32x4 b4 = i32x4{fb[set][j][0].x, fb[set][j][0].y, fb[set][j][1].x, fb[set][j][1].y};
+    acc[i][j] = MMA::run(b4, fa[set][i], acc[i][j]);   // rows = n, cols = m: the tile comes out transposed
+  };
+
+  // ---- pipeline ----------------------------------------------------------
+  // Ring of STAGES slabs.  Inside the iteration of slab t the barrier sits
+  // before the last k step: by then every wave has read all of slab t, so its
+  // slot is handed to the DMA of slab t+STAGES, and slab t+1 is known to have
+  // landed, so its first fragments are fetched under the last k step's MFMAs.
+  // The K loop is cut in three (DMA still to issue / ring draining / final
+  // slab) so the accumulators flow through straight-line code.
+
+  // k steps 0 .. KSTEPS-2 of the slab at (sa, sb): multiply register set
+  // (ks & 1) while filling the other set with step ks+1
+  auto inner_steps = [&](uint32_t sa, uint32_t sb) {
+#pragma unroll
+    for (int ks = 0; ks + 1 < C::KSTEPS; ++ks) {
+      int rd = 0;
+#pragma unroll
+      for (int x = 0; x < NMMA; ++x) {
+        mma_one(ks & 1, x);
+#pragma unroll
+        for (int q = 0; q < RPM; ++q)
+          if (rd < NREAD) { read_one((ks + 1) & 1, rd, sa, sb, ks + 1); ++rd; }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  constexpr int LAST = (C::KSTEPS - 1) & 1;   // register set holding the last k step
+  constexpr int NEXT0 = C::KSTEPS & 1;        // set that receives step 0 of the next slab
+  auto swap_sets = [&]() {                    // odd KSTEPS: the sets trade roles every slab
+    if (C::KSTEPS & 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) { i32x4 tmp = fa[0][i]; fa[0][i] = fa[1][i]; fa[1][i] = tmp; }
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) { i32x2 tmp = fb[0][j][h]; fb[0][j][h] = fb[1][j][h]; fb[1][j][h] = tmp; }
+    }
+  };
+
+  if (KT > 0) {
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s) {
+      if (s < KT) {
+        if constexpr (FAST) {
+#pragma unroll
+          for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(s));
+          dma_advance();
+        } else {
+          load_slab_generic(kt0 + s, stage_of(s));
+        }
+      }
+    }
+    if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
+    __syncthreads();
+    const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
+#pragma unroll
+    for (int r = 0; r < NREAD; ++r) read_one(0, r, sa, sb, 0);
+  }
+
+  int t = 0;
+  // (1) slabs whose slot is refilled by the DMA of slab t+STAGES
+  for (; t + STAGES < KT; ++t) {
+    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
+    inner_steps(sa, sb);
+    __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, sa);
+    const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
+    int rd = 0, dq = 0;
+#pragma unroll
+    for (int x = 0; x < NMMA; ++x) {
+      mma_one(LAST, x);
+#pragma unroll
+      for (int q = 0; q < RPM; ++q)
+        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
+      if constexpr (FAST) {
+#pragma unroll
+        for (int q = 0; q < DPM; ++q)
+          if (dq < C::LPW) { dma_op(dq, sa); ++dq; }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (FAST) dma_advance();
+    swap_sets();
+  }
+  // (2) ring draining: nothing left to issue
+  for (; t + 1 < KT; ++t) {
+    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
+    inner_steps(sa, sb);
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
+    int rd = 0;
+#pragma unroll
+    for (int x = 0; x < NMMA; ++x) {
+      mma_one(LAST, x);
+#pragma unroll
+      for (int q = 0; q < RPM; ++q)
+        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    swap_sets();
+  }
+  // (3) final slab
+  if (KT > 0) {
+    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
+    inner_steps(sa, sb);
+#pragma unroll
+    for (int x = 0; x < NMMA; ++x) mma_one(LAST, x);
+  }
+
+  // ---- epilogue ------------------------------------------------------------
+  // The MFMA was issued with the B fragment as its row operand, so the tile it
+  // returns is C^T: lane l owns output row m = l % MI and, per group of four
+  // accumulator registers, four consecutive columns n.  Four columns make one
+  // 8-byte (16-bit out) or 16-byte (32-bit out) store, and a gate/linear pair
+  // of the GLU epilogue sits inside one lane.
+  const int64_t gm_base = m0 + wy * C::WTM + (lane % MI);
+  const int64_t gn_base = n0 + wx * C::WTN + (lane / MI) * 4;
+  if (p.split_k > 1) {
+    acc_s* ws = (acc_s*)p.ws + (int64_t)split * p.m * p.n;
+    epilogue_store<T, C, acc_s, EPI_NONE>(acc, (uint8_t*)ws, gm_base, gn_base, p.m, p.n, p.n, 1, (p.n & 3) == 0, 0);
+  } else if (p.epilogue == EPI_NONE) {
+    epilogue_store<T, C, typename OutOf<T>::type, EPI_NONE>(acc, p.c, gm_base, gn_base, p.m, p.n, p.scm, p.scn,
+                                                            p.c_vec_ok, 0);
+  } else {
+    epilogue_store<T, C, typename OutOf<T>::type, 1>(acc, p.c, gm_base, gn_base, p.m, p.n, p.scm, p.scn, p.c_vec_ok,
+                                                     p.epilogue);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// split-K second pass: sum the partials in a fixed order, then apply the
+// epilogue.  One thread per output element.
+// ---------------------------------------------------------------------------
+template <class ACC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const ACC* __restrict__ ws, uint8_t* c, int64_t m, int64_t n,
+                                                            int64_t scm, int64_t scn, int split_k, int epilogue,
+                                                            int out_dtype) {
+  const int64_t ncols = epilogue == EPI_NONE ? n : n / 2;
+  const int64_t total = m * ncols;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    int64_t gm = idx / ncols, gc = idx % ncols;
+    if (epilogue == EPI_NONE) {
+      ACC s = 0;
+      for (int z = 0; z < split_k; ++z) s += ws[((int64_t)z * m + gm) * n + gc];
+      store_out<ACC>(c, gm * scm + gc * scn, s, out_dtype);
+    } else {
+      float g = 0.f, l = 0.f;
+      for (int z = 0; z < split_k; ++z) {
+        g += (float)ws[((int64_t)z * m + gm) * n + 2 * gc];
+        l += (float)ws[((int64_t)z * m + gm) * n + 2 * gc + 1];
+      }
+      store_out<float>(c, gm * scm + gc * scn, glu_gate(g, epilogue) * l, out_dtype);
+    }
+  }
+}
+
+}  // namespace tnx

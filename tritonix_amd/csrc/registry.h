@@ -1,0 +1,36 @@
+// Table of compiled tile kernels.  Each generated instance file contributes
+// one array of KernelEntry; capi.hip looks a tile config up in the union.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "gemm_tile.h"
+
+namespace tnx {
+
+typedef hipError_t (*launch_fn)(const GemmParams& p, unsigned grid, hipStream_t stream);
+
+struct KernelEntry {
+  int dtype, bm, bn, bk, nw, stages;
+  int lds_bytes;
+  launch_fn fast;     // DMA loader: row-major, 16-byte aligned, k % bk == 0
+  launch_fn generic;  // element-wise loader: any strides / ragged k; may be null
+};
+
+struct KernelGroup {
+  KernelEntry* entries;
+  int count;
+};
+
+template <class T, class C, bool FAST>
+hipError_t launch_tile(const GemmParams& p, unsigned grid, hipStream_t stream) {
+  static_assert(C::VALID, "tile configuration is not buildable");
+  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST>), dim3(grid), dim3(C::THREADS), 0, stream, p);
+  return hipGetLastError();
+}
+
+#define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
+  {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
+   &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \
+   GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr}
+
+}  // namespace tnx
