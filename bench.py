@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the tiled-GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune] [--no-extras] [--no-cpu]
+
+A step is one launch of the headline workload -- the bf16 8192^3 GEMM
+(row-major A and B, fp32 accumulate, bf16 out, non-split tiled kernel with
+the group-M swizzle) -- through the C ABI, operands resident in HBM.  Prints
+one JSON line: whole-job TFLOP/s over the K timed steps, the roofline record
+of the kernel (algorithmic flops / mean per-launch duration from HIP events
+on the launch stream), the CPU baseline (torch fp32 matmul on the host
+cores, bounded sample) and, under "per_config", the other four benchmark
+configurations measured the same way.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+PEAK = {"bf16": 2516.6, "f16": 2516.6, "i8": 5033.2}     # dense MFMA TFLOP/s (TOP/s), MI355X
+HBM_PEAK_GBS = 8000.0
+
+# measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the headline kernel; see profiles/
+TRAFFIC_BYTES_C2 = None
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--tune", action="store_true", help="run the grid tuner for each workload instead of the built-in tiles")
+    ap.add_argument("--no-extras", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return ap.parse_args()
+
+
+def event_times(fn, n):
+    """Per-launch durations in ms from HIP events recorded on torch's current stream (the launch stream)."""
+    import torch
+
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    for i in range(n):
+        starts[i].record()
+        fn(i)
+        stops[i].record()
+    torch.cuda.synchronize()
+    return [s.elapsed_time(e) for s, e in zip(starts, stops)]
+
+
+def pick_config(kernel, launcher, a, b, tune, split=False):
+    from tritonix_amd.ops.matmul import default_config
+
+    if tune:
+        cfg = kernel.tune(launcher, warmup=5, rep=20)
+        if cfg is not None:
+            return cfg
+    return default_config(a, b, split=split)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X: no HIP device is visible", file=sys.stderr)
+        return 2
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import oracle                                  # inputs + CPU baseline only; never on the measured path
+    from tritonix_amd import _C
+    import importlib
+
+    mm = importlib.import_module("tritonix_amd.ops.matmul")
+    sg = importlib.import_module("tritonix_amd.ops.swiglu")
+
+    _C.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    # ---- headline: C2 --------------------------------------------------------------
+    a_cpu, b_cpu = oracle.make_inputs("C2")
+    a, b = a_cpu.to(dev), b_cpu.to(dev)
+    m, k = a.shape
+    n = b.shape[1]
+    flops = 2.0 * m * n * k
+    cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+    c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
+    grid = (-(-m // cfg["block_m"]), -(-n // cfg["block_n"]))
+
+    def step(_i=0):
+        mm.matmul_kernel[grid](a, b, c, m, n, k, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0),
+                               c.stride(1), **cfg)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = flops * args.steps / wall / 1e12
+
+    durs = event_times(step, max(10, min(args.steps, 100)))
+    kern_ms = sum(durs) / len(durs)
+    achieved = flops / kern_ms / 1e9
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK["bf16"], "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK["bf16"], 4), "traffic": TRAFFIC_BYTES_C2,
+                "kernel_ms": round(kern_ms, 4), "kernel_ms_min": round(min(durs), 4)}
+
+    # parity of what was just timed, on a sample of rows (the oracle is the checker, not the thing measured)
+    rows = torch.arange(0, m, 517)
+    ok, maxerr, rel = oracle.within_tolerance(c[rows.to(dev)], oracle.reference_matmul(a_cpu[rows], b_cpu))
+
+    # ---- CPU baseline: the reference's "pytorch" backend restated on the host ---------
+    cpu = None
+    if not args.no_cpu:
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        rows_n = 2048                                   # bounded sample: first 2048 rows of A against all of B
+        af, bf = a_cpu[:rows_n].float(), b_cpu.float()
+        torch.matmul(af[:256], bf)                      # warm-up
+        reps, ts = 0, []
+        t_start = time.perf_counter()
+        while reps < 3 and time.perf_counter() - t_start < 30:
+            t1 = time.perf_counter()
+            torch.matmul(af, bf)
+            ts.append(time.perf_counter() - t1)
+            reps += 1
+        med = sorted(ts)[len(ts) // 2]
+        cpu = {"value": round(2.0 * rows_n * n * k / med / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": f"torch fp32 CPU matmul, first {rows_n} of {m} rows of A x full B, median of {reps}"}
+
+    out = {
+        "metric": "TFLOP/s + % of dense MFMA peak, bf16 GEMM 8192^3 on 1xMI355X",
+        "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C2: bf16 GEMM M=N=K=8192, A,B ~ N(0,1)/sqrt(K) seed 2, row-major, fp32 acc, bf16 out",
+                   "tile": cfg},
+        "pct_of_peak": round(100 * value / PEAK["bf16"], 2),
+        "roofline": roofline, "cpu_baseline": cpu,
+        "parity": {"ok": bool(ok), "max_abs_err": maxerr, "max_err_over_max_ref": rel, "rows_checked": int(rows.numel())},
+    }
+    del a, b, c
+
+    # ---- the other configurations ------------------------------------------------------
+    if not args.no_extras:
+        out["per_config"] = extras(torch, dev, oracle, mm, sg, args)
+    print(json.dumps(out))
+    return 0 if ok else 1
+
+
+def extras(torch, dev, oracle, mm, sg, args):
+    from tritonix_amd.kernel import out_dtype_for
+
+    res = {}
+    reps = 30
+
+    def measure(name, fn, flops, bytes_, dt, bound, nrot=1):
+        for i in range(5):
+            fn(i % nrot)
+        torch.cuda.synchronize()
+        durs = event_times(lambda i: fn(i % nrot), reps)
+        ms = sum(durs) / len(durs)
+        r = {"kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "gbs": round(bytes_ / ms / 1e6, 1)}
+        if bound == "mfma":
+            r["roofline"] = {"bound": "mfma", "achieved": r["tflops"], "peak": PEAK[dt], "unit": "TFLOP/s",
+                             "frac": round(r["tflops"] / PEAK[dt], 4)}
+        elif bound == "hbm":
+            r["roofline"] = {"bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(r["gbs"] / HBM_PEAK_GBS, 4)}
+        res[name] = r
+        return r
+
+    # C1: latency-bound, report only
+    a, b = (t.to(dev) for t in oracle.make_inputs("C1"))
+    cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+    c = torch.empty((1024, 768), device=dev, dtype=torch.float16)
+    measure("C1", lambda i: mm.matmul_kernel[(1,)](a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg),
+            805306368, 3407872, "f16", None)["tile"] = cfg
+
+    # C3: B is streamed from HBM: rotate distinct copies of B so that none is served from the 256 MiB Infinity Cache
+    a_cpu, b_cpu = oracle.make_inputs("C3")
+    a = a_cpu.to(dev)
+    nrot = 4
+    bs = [b_cpu.to(dev).clone() for _ in range(nrot)]
+    cfg = pick_config(mm.gemm_splitk_kernel, lambda c: mm._launch_splitk(a, bs[0], c), a, bs[0], args.tune, split=True)
+    c = torch.empty((16, 4096), device=dev, dtype=torch.bfloat16)
+    r = measure("C3", lambda i: mm.gemm_splitk_kernel[(1,)](a, bs[i], c, 16, 4096, 14336, 14336, 1, 4096, 1, 4096, 1,
+                                                            **cfg),
+                1879048192, 118030336, "bf16", "hbm", nrot=nrot)
+    r["tile"] = cfg
+    r["note"] = f"{nrot} distinct copies of B rotated ({nrot * 117} MB > 256 MB Infinity Cache); time includes the split-K reduce kernel"
+    ok, _, rel = oracle.within_tolerance(c, oracle.reference_matmul(a_cpu, b_cpu))
+    r["parity_ok"] = bool(ok)
+    del bs
+
+    # C4: fused GLU, both activations
+    x_cpu, w_cpu = oracle.make_inputs("C4")
+    x, w = x_cpu.to(dev), w_cpu.to(dev)
+    cfg = pick_config(sg.glu_kernel, lambda c: sg._launch_glu(x, w, c, "silu"), x, w, args.tune)
+    z = torch.empty((4096, 14336), device=dev, dtype=torch.bfloat16)
+    for act in ("silu", "sigmoid"):
+        measure(f"C4_{act}", lambda i: sg.glu_kernel[(1,)](x, w, z, 4096, 28672, 4096, 4096, 1, 28672, 1, 14336, 1,
+                                                           activation=act, **cfg),
+                962072674304, 385875968, "bf16", "mfma")["tile"] = cfg
+    rows = torch.arange(0, 4096, 409)
+    res["C4_sigmoid"]["parity_ok"] = bool(oracle.within_tolerance(z[rows.to(dev)],
+                                                                  oracle.reference_glu(x_cpu[rows], w_cpu, "sigmoid"))[0])
+    del x, w, z
+
+    # C5: int8 -> int32
+    a_cpu, b_cpu = oracle.make_inputs("C5")
+    a, b = a_cpu.to(dev), b_cpu.to(dev)
+    cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+    c = torch.empty((8192, 8192), device=dev, dtype=torch.int32)
+    r = measure("C5", lambda i: mm.matmul_kernel[(1,)](a, b, c, 8192, 8192, 8192, 8192, 1, 8192, 1, 8192, 1, **cfg),
+                1099511627776, 402653184, "i8", "mfma")
+    r["tile"] = cfg
+    rows = torch.arange(0, 8192, 1021)
+    r["bit_exact"] = bool(torch.equal(c[rows.to(dev)].cpu(), oracle.reference_matmul(a_cpu[rows], b_cpu)))
+    return res
+
+
+if __name__ == "__main__":
+    sys.exit(main())

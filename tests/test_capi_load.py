@@ -1,0 +1,114 @@
+"""The C-ABI library loads, exports every symbol include/tritonix_hip.h declares, and its host-only entry points
+answer without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from tritonix_amd import _C
+from tritonix_amd.testing import LDS_LIMIT_BYTES, OutOfResources
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def args(**kw):
+    g = _C.GemmArgs()
+    base = dict(m=512, n=512, k=512, stride_am=512, stride_ak=1, stride_bk=512, stride_bn=1, stride_cm=512,
+                stride_cn=1, in_dtype=_C.BF16, out_dtype=_C.BF16, block_m=128, block_n=128, block_k=64, group_m=8,
+                split_k=1, num_stages=2, num_warps=4, epilogue=_C.EPI_NONE)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(g, k, v)
+    return g
+
+
+def test_library_is_built_and_exports_the_header():
+    lib = _C.load()
+    header = open(os.path.join(ROOT, "include", "tritonix_hip.h")).read()
+    declared = set(re.findall(r"\b(tnx_[a-z_0-9]+)\s*\(", header)) - {"tnx_gemm_args"}
+    assert declared == set(_C.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.tnx_version() == int(re.search(r"#define TNX_VERSION (\d+)", header).group(1))
+    assert int(re.search(r"#define TNX_LDS_LIMIT_BYTES (\d+)", header).group(1)) == LDS_LIMIT_BYTES
+
+
+def test_struct_layout_matches_the_header_field_order():
+    header = open(os.path.join(ROOT, "include", "tritonix_hip.h")).read()
+    start = header.index("typedef struct tnx_gemm_args {") + len("typedef struct tnx_gemm_args {")
+    body = header[start:header.index("} tnx_gemm_args;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl or decl.startswith("typedef"):
+            continue
+        decl = re.sub(r"^(const\s+)?(void|int64_t|int32_t|size_t)\s*\*?", "", decl)
+        names += [n.strip(" *") for n in decl.split(",")]
+    assert names == [f[0] for f in _C.GemmArgs._fields_]
+    assert ctypes.sizeof(_C.GemmArgs) == 3 * 8 + 9 * 8 + 10 * 4 + 8 + 8 + 8
+
+
+def test_lds_bytes_is_host_arithmetic():
+    lib = _C.load()
+    assert lib.tnx_gemm_lds_bytes(ctypes.byref(args())) == 2 * (128 * 64 + 64 * 128) * 2
+    assert lib.tnx_gemm_lds_bytes(ctypes.byref(args(block_m=256, block_n=256, num_stages=2))) == 131072
+    assert lib.tnx_gemm_lds_bytes(ctypes.byref(args(in_dtype=_C.I8, out_dtype=_C.I32, block_k=128))) == 65536
+    assert lib.tnx_gemm_lds_bytes(ctypes.byref(args(block_m=0))) == -1
+
+
+def test_supported_status_codes_and_python_exceptions():
+    lib = _C.load()
+    ok = args()
+    assert lib.tnx_gemm_supported(ctypes.byref(ok)) == _C.OK
+    too_big = args(block_m=256, block_n=256, num_stages=3)             # 196608 bytes of LDS
+    assert lib.tnx_gemm_supported(ctypes.byref(too_big)) == _C.E_LDS
+    with pytest.raises(OutOfResources) as ei:
+        _C.raise_for_status(_C.E_LDS, too_big)
+    assert (ei.value.required, ei.value.limit, ei.value.name) == (196608, 163840, "shared memory")
+    assert "Required: 196608" in str(ei.value)
+    odd = args(block_m=96)
+    assert lib.tnx_gemm_supported(ctypes.byref(odd)) == _C.E_UNSUPPORTED
+    with pytest.raises(ValueError):
+        _C.raise_for_status(_C.E_UNSUPPORTED, odd)
+    assert lib.tnx_gemm_supported(ctypes.byref(args(out_dtype=_C.F16))) == _C.E_UNSUPPORTED   # bf16 in, f16 out
+    assert lib.tnx_gemm_supported(ctypes.byref(args(epilogue=_C.EPI_GLU_SILU, n=511))) == _C.E_UNSUPPORTED
+    assert lib.tnx_gemm_supported(ctypes.byref(args(m=-1))) == _C.E_INVALID
+    assert lib.tnx_gemm_supported(ctypes.byref(args(in_dtype=9))) == _C.E_INVALID
+    assert lib.tnx_gemm_supported(None) == _C.E_INVALID
+    with pytest.raises(RuntimeError):
+        _C.raise_for_status(_C.E_HIP, ok)
+    assert _C.strerror(_C.OK) == "ok" and "LDS" in _C.strerror(_C.E_LDS)
+
+
+def test_ragged_layouts_need_a_generic_kernel():
+    lib = _C.load()
+    # k not a multiple of block_k: only tiles built with the element-wise loader accept it
+    assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500))) == _C.OK          # 128x128x64 w4 s2
+    assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500, num_stages=3))) == _C.E_UNSUPPORTED
+    # column-major B
+    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=512))) == _C.OK
+    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=512, num_warps=8))) == _C.E_UNSUPPORTED
+
+
+def test_workspace_bytes_and_default_config():
+    lib = _C.load()
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args())) == 0
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=16, n=4096, k=14336, split_k=8))) == 8 * 16 * 4096 * 4
+    g = args(m=8192, n=8192, k=8192)
+    assert lib.tnx_gemm_default_config(ctypes.byref(g)) == _C.OK
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK
+    g = args(m=16, n=4096, k=14336)
+    lib.tnx_gemm_default_config(ctypes.byref(g))
+    assert g.split_k >= 4 and lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK
+    g = args(in_dtype=_C.I8, out_dtype=_C.I32, m=8192, n=8192, k=8192)
+    lib.tnx_gemm_default_config(ctypes.byref(g))
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK
+
+
+def test_kernel_table_lists_every_dtype():
+    names = _C.kernel_names()
+    assert len(names) == _C.load().tnx_kernel_count() > 0
+    assert {n.split()[0] for n in names} == {"bf16", "f16", "i8"}
+    assert _C.load().tnx_kernel_name(len(names)) is None

@@ -1,0 +1,130 @@
+"""The reference's own GPU tests (tests/test_matmul.py: correctness, forced backends, cached winner) on the
+HIP path, plus the ops it never tested: split-K, GLU, int8."""
+import pytest
+import torch
+
+import oracle
+import tritonix_amd
+import importlib
+
+mm = importlib.import_module("tritonix_amd.ops.matmul")   # the module; `tritonix_amd.ops.matmul` the attribute is the dispatcher
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def short_tuning(monkeypatch):
+    monkeypatch.setitem(mm.TUNE_OPTIONS, "warmup", 1)
+    monkeypatch.setitem(mm.TUNE_OPTIONS, "rep", 3)
+
+
+def close(ref, out):
+    # the reference's own bar (tests/test_matmul.py:18-20)
+    return torch.allclose(ref.float(), out.float(), atol=1.0, rtol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (1024, 2048, 512), (2048, 2048, 2048)])
+def test_matmul_correctness(device, M, N, K):
+    g = torch.Generator("cpu").manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).half().to(device)
+    b = torch.randn(K, N, generator=g).half().to(device)
+    out = tritonix_amd.triton_matmul(a, b)
+    assert close(torch.matmul(a, b), out), f"max diff: {(torch.matmul(a, b) - out).abs().max()}"
+    ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
+    assert ok and rel <= 1e-2
+    assert (M, N, K, torch.float16) in mm._matmul_cfg
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (2048, 2048, 2048)])
+def test_dispatch_correctness(device, M, N, K):
+    a = torch.randn(M, K, device=device, dtype=torch.float16)
+    b = torch.randn(K, N, device=device, dtype=torch.float16)
+    ref = torch.matmul(a, b)
+    with tritonix_amd.matmul.force_backend("triton"):
+        tri = tritonix_amd.matmul(a, b)
+    with tritonix_amd.matmul.force_backend("pytorch"):
+        pt = tritonix_amd.matmul(a, b)
+    assert close(ref, tri) and close(ref, pt)
+
+
+def test_dispatch_caches_winner(device):
+    matmul = tritonix_amd.matmul
+    matmul.clear_cache()
+    a = torch.randn(1024, 1024, device=device, dtype=torch.float16)
+    b = torch.randn(1024, 1024, device=device, dtype=torch.float16)
+    out1 = matmul(a, b)
+    assert len(matmul.cache) == 1
+    assert list(matmul.cache.values())[0] in ("triton", "pytorch")
+    assert list(matmul.cache)[0] == (1024, 1024, "torch.float16", 1024, 1024, "torch.float16")
+    out2 = matmul(a, b)
+    assert torch.allclose(out1.float(), out2.float(), atol=1.0, rtol=1e-2)
+
+
+def test_tune_entry_point_with_a_user_launcher(device):
+    # the flow of examples/tune_matmul.py: the caller writes the launcher and gets a config dict back
+    a = torch.randn(512, 1024, device=device, dtype=torch.bfloat16)
+    b = torch.randn(1024, 768, device=device, dtype=torch.bfloat16)
+    kernel = tritonix_amd.matmul_kernel
+
+    def launcher(cfg):
+        c = torch.empty((512, 768), device=device, dtype=a.dtype)
+        grid = ((512 + cfg["block_m"] - 1) // cfg["block_m"], (768 + cfg["block_n"] - 1) // cfg["block_n"])
+        kernel[grid](a, b, c, 512, 768, 1024, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0),
+                     c.stride(1), **cfg)
+        return c
+
+    best = kernel.tune(launcher, method="grid", warmup=1, rep=3, max_configs=12)
+    assert set(best) == set(kernel.space)
+    ok, _, _ = oracle.within_tolerance(launcher(best), oracle.reference_matmul(a, b))
+    assert ok
+
+
+def test_matmul_splitk(device):
+    a, b = oracle.make_inputs("C3", scale_down=2)
+    out = tritonix_amd.matmul_splitk(a.to(device), b.to(device))
+    ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
+    assert ok and rel <= 1e-2
+    assert mm._splitk_cfg[(16, 2048, 7168, 4, torch.bfloat16)]["split_k"] >= 2
+
+
+def test_glu_and_swiglu_wrappers(device):
+    x, w12 = oracle.make_inputs("C4", scale_down=16)
+    xd, wd = x.to(device), w12.to(device)
+    z = tritonix_amd.swiglu(xd, wd)
+    assert z.shape == (x.shape[0], w12.shape[1] // 2) and z.dtype == torch.bfloat16
+    assert oracle.within_tolerance(z, oracle.reference_glu(x, w12, "silu"))[0]
+    assert oracle.within_tolerance(tritonix_amd.glu(xd, wd, activation="sigmoid"),
+                                   oracle.reference_glu(x, w12, "sigmoid"))[0]
+    assert torch.equal(tritonix_amd.fused_glu(xd, wd), z)
+    from tritonix_amd.ops.swiglu import interleave_weights
+
+    w1, w2 = w12[:, 0::2].contiguous(), w12[:, 1::2].contiguous()
+    assert torch.equal(interleave_weights(w1, w2), w12)
+    with pytest.raises(ValueError):
+        tritonix_amd.glu(xd, wd[:, :-1])
+
+
+def test_int8_through_the_dispatcher(device):
+    a, b = oracle.make_inputs("C5", scale_down=16)
+    out = tritonix_amd.matmul(a.to(device), b.to(device))       # torch has no int8 GPU matmul: "pytorch" drops out
+    assert out.dtype == torch.int32
+    assert torch.equal(out.cpu(), oracle.reference_matmul(a, b))
+
+
+def test_default_config_path(device, monkeypatch):
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    mm._matmul_cfg.clear()
+    a, b = oracle.make_inputs("C2", scale_down=4)
+    out = tritonix_amd.triton_matmul(a.to(device), b.to(device))
+    assert oracle.within_tolerance(out, oracle.reference_matmul(a, b))[0]
+
+
+def test_do_bench_returns_sane_numbers(device):
+    from tritonix_amd.testing import do_bench
+
+    a = torch.randn(2048, 2048, device=device, dtype=torch.bfloat16)
+    ms = do_bench(lambda: torch.matmul(a, a), warmup=2, rep=10)
+    tflops = 2 * 2048 ** 3 / ms / 1e9
+    assert 0 < tflops < 1e4
+    q = do_bench(lambda: torch.matmul(a, a), warmup=2, rep=10, quantiles=[0.5, 0.2, 0.8])
+    assert len(q) == 3 and q[1] <= q[0] <= q[2]

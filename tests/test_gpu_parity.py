@@ -1,0 +1,226 @@
+"""GPU parity: the HIP kernels, called through the C ABI (HipKernel -> tnx_gemm), against the CPU oracle on
+the same seeded inputs.  Integer work must be bit-exact; floating point must satisfy
+|out - ref| <= 1e-2*|ref| + 1e-2*rms(ref) and max|out-ref|/max|ref| <= 1e-2 against the fp32 CPU matmul."""
+import pytest
+import torch
+
+import oracle
+from tritonix_amd.kernel import cdiv, out_dtype_for
+from tritonix_amd.ops.matmul import gemm_splitk_kernel, matmul_kernel
+from tritonix_amd.ops.swiglu import glu_kernel
+from tritonix_amd.testing import OutOfResources
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-2
+
+
+def cfg(bm, bn, bk, nw, st, gm=8, **extra):
+    return dict(block_m=bm, block_n=bn, block_k=bk, group_m=gm, num_stages=st, num_warps=nw, **extra)
+
+
+def run(kernel, a, b, c, config, **kw):
+    m, k = a.shape
+    n = b.shape[1]
+    grid = (cdiv(m, config["block_m"]), cdiv(n, config["block_n"]))
+    kernel[grid](a, b, c, m, n, k, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                 **config, **kw)
+    torch.cuda.synchronize()
+    return c
+
+
+def gemm(a, b, config, kernel=matmul_kernel):
+    c = torch.full((a.shape[0], b.shape[1]), 7, device=a.device, dtype=out_dtype_for(a.dtype))
+    return run(kernel, a, b, c, config)
+
+
+def check_fp(out, ref):
+    ok, maxerr, rel = oracle.within_tolerance(out, ref, REL)
+    assert ok, f"outside tolerance: max err {maxerr}, max err / max|ref| {rel}"
+    assert rel <= REL
+
+
+F16_TILES = [cfg(128, 128, 64, 4, 2), cfg(128, 128, 64, 4, 3), cfg(256, 256, 64, 4, 2), cfg(64, 128, 64, 4, 3, gm=4),
+             cfg(128, 128, 64, 8, 2), cfg(256, 256, 64, 8, 2), cfg(64, 128, 64, 8, 3)]
+
+
+# ---- C1: fp16 1024x512 @ 512x768, full size ------------------------------------------
+@pytest.mark.parametrize("config", F16_TILES, ids=lambda c: "x".join(str(v) for v in c.values()))
+def test_c1_fp16_full_size(device, config):
+    a, b = oracle.make_inputs("C1")
+    out = gemm(a.to(device), b.to(device), config)
+    assert out.dtype == torch.float16
+    check_fp(out, oracle.reference_matmul(a, b))
+
+
+# ---- C2: bf16 square ------------------------------------------------------------------
+@pytest.mark.parametrize("config", [cfg(256, 256, 64, 4, 2), cfg(256, 256, 64, 8, 2), cfg(128, 128, 64, 4, 3)],
+                         ids=lambda c: "x".join(str(v) for v in c.values()))
+def test_c2_bf16_square_1024(device, config):
+    a, b = oracle.make_inputs("C2", scale_down=8)
+    check_fp(gemm(a.to(device), b.to(device), config), oracle.reference_matmul(a, b))
+
+
+def test_c2_bf16_full_size_rows_and_linearity(device):
+    a, b = oracle.make_inputs("C2")
+    ad, bd = a.to(device), b.to(device)
+    config = cfg(256, 256, 64, 4, 2)
+    out = gemm(ad, bd, config)
+    rows = torch.tensor([0, 1, 255, 256, 4095, 4096, 8190, 8191] + list(range(1000, 8000, 500)))
+    check_fp(out[rows.to(device)], oracle.reference_matmul(a[rows], b))
+    # scaling an operand by a power of two scales every product and partial sum exactly
+    out2 = gemm(ad * 2, bd, config)
+    assert torch.equal(out2, out * 2)
+    # and a second launch reproduces the first bit for bit
+    assert torch.equal(gemm(ad, bd, config), out)
+
+
+# ---- C3: skinny split-K ---------------------------------------------------------------
+@pytest.mark.parametrize("split_k", [2, 4, 8, 16])
+def test_c3_splitk_full_size(device, split_k):
+    a, b = oracle.make_inputs("C3")
+    ad, bd = a.to(device), b.to(device)
+    config = cfg(64, 128, 64, 4, 3, split_k=split_k)
+    out = gemm(ad, bd, config, kernel=gemm_splitk_kernel)
+    assert out.shape == (16, 4096) and out.dtype == torch.bfloat16
+    check_fp(out, oracle.reference_matmul(a, b))
+    # workspace partials summed in a fixed order: run-to-run identical, no atomics
+    assert torch.equal(gemm(ad, bd, config, kernel=gemm_splitk_kernel), out)
+
+
+def test_splitk_matches_non_split_within_rounding(device):
+    a, b = oracle.make_inputs("C3", scale_down=4)
+    ad, bd = a.to(device), b.to(device)
+    plain = gemm(ad, bd, cfg(64, 128, 64, 4, 3))
+    split = gemm(ad, bd, cfg(64, 128, 64, 4, 3, split_k=7), kernel=gemm_splitk_kernel)   # 56 slabs / 7
+    ref = oracle.reference_matmul(a, b)
+    check_fp(split, ref)
+    check_fp(plain, ref)
+    # more splits than K slabs: the empty splits must contribute zeros
+    tiny_a, tiny_b = ad[:, :128].contiguous(), bd[:128].contiguous()
+    check_fp(gemm(tiny_a, tiny_b, cfg(64, 128, 64, 4, 3, split_k=16), kernel=gemm_splitk_kernel),
+             oracle.reference_matmul(tiny_a, tiny_b))
+
+
+# ---- C4: fused GLU --------------------------------------------------------------------
+@pytest.mark.parametrize("activation", ["silu", "sigmoid", "identity"])
+@pytest.mark.parametrize("config", [cfg(256, 256, 64, 4, 2), cfg(128, 128, 64, 4, 3), cfg(128, 128, 64, 8, 2)],
+                         ids=lambda c: "x".join(str(v) for v in c.values()))
+def test_c4_glu_scaled(device, activation, config):
+    x, w12 = oracle.make_inputs("C4", scale_down=8)     # x[512,512], w12[512,3584]
+    z = torch.full((x.shape[0], w12.shape[1] // 2), 7, device=device, dtype=torch.bfloat16)
+    run(glu_kernel, x.to(device), w12.to(device), z, config, activation=activation)
+    check_fp(z, oracle.reference_glu(x, w12, activation))
+
+
+def test_c4_glu_full_size_rows(device):
+    x, w12 = oracle.make_inputs("C4")
+    xd, wd = x.to(device), w12.to(device)
+    rows = torch.tensor([0, 255, 256, 2047, 2048, 4095] + list(range(100, 4000, 390)))
+    for act in ("silu", "sigmoid"):
+        z = torch.empty((4096, 14336), device=device, dtype=torch.bfloat16)
+        run(glu_kernel, xd, wd, z, cfg(256, 256, 64, 4, 2), activation=act)
+        check_fp(z[rows.to(device)], oracle.reference_glu(x[rows], w12, act))
+
+
+# ---- C5: int8 -> int32, bit-exact -----------------------------------------------------
+@pytest.mark.parametrize("config", [cfg(256, 256, 128, 4, 2), cfg(128, 128, 128, 4, 2), cfg(256, 256, 128, 8, 2),
+                                    cfg(64, 128, 128, 4, 3)], ids=lambda c: "x".join(str(v) for v in c.values()))
+def test_c5_int8_exact_1024(device, config):
+    a, b = oracle.make_inputs("C5", scale_down=8)
+    out = gemm(a.to(device), b.to(device), config)
+    assert out.dtype == torch.int32
+    assert torch.equal(out.cpu(), oracle.reference_matmul(a, b))
+
+
+def test_c5_int8_full_size_rows_exact(device):
+    a, b = oracle.make_inputs("C5")
+    out = gemm(a.to(device), b.to(device), cfg(256, 256, 128, 4, 2))
+    rows = torch.tensor([0, 255, 256, 4095, 4096, 8191] + list(range(77, 8000, 997)))
+    assert torch.equal(out[rows.to(device)].cpu(), oracle.reference_matmul(a[rows], b))
+    # a checksum over the whole result: sum_j C[i,j] == A[i,:] . (B @ 1)
+    colsum = b.double().sum(dim=1)
+    assert torch.equal(out.sum(dim=1, dtype=torch.int64).cpu(), (a.double() @ colsum).to(torch.int64))
+
+
+def test_int8_extremes(device):
+    a = torch.full((64, 8192), -127, dtype=torch.int8)
+    b = torch.full((8192, 128), -127, dtype=torch.int8)
+    out = gemm(a.to(device), b.to(device), cfg(64, 128, 128, 4, 3))
+    assert int(out.min()) == int(out.max()) == 8192 * 127 * 127
+
+
+# ---- edges: ragged shapes, strides, tiny and empty problems ----------------------------
+GENERIC = cfg(128, 128, 64, 4, 2)       # built with the element-wise loader as well
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 8, 64), (16, 24, 40), (100, 264, 200), (129, 257, 65),
+                                   (300, 264, 192), (37, 1000, 333)])
+def test_ragged_shapes_bf16(device, m, n, k):
+    g = torch.Generator("cpu").manual_seed(m * 131 + n * 17 + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    b = torch.randn(k, n, generator=g).bfloat16()
+    check_fp(gemm(a.to(device), b.to(device), GENERIC), oracle.reference_matmul(a, b))
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 7, 3), (33, 17, 100)])
+def test_tiny_shapes_against_the_tile_walking_oracle(device, m, n, k):
+    g = torch.Generator("cpu").manual_seed(9)
+    a = torch.randn(m, k, generator=g).half()
+    b = torch.randn(k, n, generator=g).half()
+    walk = torch.from_numpy(oracle.tiled_matmul(a.float().numpy(), b.float().numpy(), 32, 32, 16, 4))
+    check_fp(gemm(a.to(device), b.to(device), GENERIC), walk)
+    ai = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8)
+    bi = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+    got = gemm(ai.to(device), bi.to(device), cfg(128, 128, 128, 4, 2))
+    assert torch.equal(got.cpu(), torch.from_numpy(oracle.tiled_matmul_i8(ai.numpy(), bi.numpy())))
+
+
+def test_strided_operands_and_output(device):
+    g = torch.Generator("cpu").manual_seed(11)
+    at = torch.randn(192, 160, generator=g).bfloat16()       # use a = at.T (column-major A)
+    bt = torch.randn(136, 192, generator=g).bfloat16()       # use b = bt.T (column-major B)
+    a, b = at.t(), bt.t()
+    ref = oracle.reference_matmul(a, b)
+    check_fp(gemm(a.to(device).t().contiguous().t(), b.to(device), GENERIC), ref)   # contiguous a, strided b
+    ad, bd = at.to(device).t(), bt.to(device).t()
+    assert ad.stride() == (1, 160) and bd.stride() == (1, 192)
+    check_fp(gemm(ad, bd, GENERIC), ref)
+    # output with a row pitch and a column step
+    buf = torch.zeros(160, 2 * 136 + 6, device=device, dtype=torch.bfloat16)
+    c = buf[:, 3:3 + 2 * 136:2]
+    run(matmul_kernel, ad, bd, c, GENERIC)
+    check_fp(c, ref)
+    assert float(buf[:, :3].abs().sum()) == 0 and float(buf[:, 4::2].abs().sum()) == 0
+    # row-major operands whose rows are padded stay on the fast loader
+    wide_a = torch.zeros(256, 512 + 64, device=device, dtype=torch.bfloat16)
+    wide_b = torch.zeros(512, 384 + 8, device=device, dtype=torch.bfloat16)
+    a2 = torch.randn(256, 512, generator=g).bfloat16()
+    b2 = torch.randn(512, 384, generator=g).bfloat16()
+    wide_a[:, :512] = a2.to(device)
+    wide_b[:, :384] = b2.to(device)
+    check_fp(gemm(wide_a[:, :512], wide_b[:, :384], cfg(128, 128, 64, 4, 3)), oracle.reference_matmul(a2, b2))
+
+
+def test_empty_problems(device):
+    a = torch.zeros(0, 64, device=device, dtype=torch.bfloat16)
+    b = torch.zeros(64, 32, device=device, dtype=torch.bfloat16)
+    assert gemm(a, b, GENERIC).shape == (0, 32)
+    # k == 0: the product is all zeros
+    a = torch.zeros(8, 0, device=device, dtype=torch.bfloat16)
+    b = torch.zeros(0, 16, device=device, dtype=torch.bfloat16)
+    assert float(gemm(a, b, GENERIC).abs().sum()) == 0
+
+
+def test_error_mapping_on_launch(device):
+    a = torch.zeros(256, 256, device=device, dtype=torch.bfloat16)
+    with pytest.raises(OutOfResources):
+        gemm(a, a, cfg(256, 256, 64, 4, 3))           # 196608 B of LDS: rejected before any launch
+    with pytest.raises(ValueError):
+        gemm(a, a, cfg(96, 128, 64, 4, 2))            # no such tile
+    with pytest.raises(ValueError):
+        gemm(a[:, :200], a[:200], cfg(128, 128, 64, 4, 3))   # ragged K on a DMA-only tile
+    with pytest.raises(ValueError):
+        gemm(a.float(), a.float(), GENERIC)
+    with pytest.raises(ValueError):
+        gemm(a.cpu(), a.cpu(), GENERIC)

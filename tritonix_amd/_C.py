@@ -1,0 +1,108 @@
+"""ctypes binding of libtritonix_hip.so (the C ABI declared in include/tritonix_hip.h).
+
+The library is built ahead of time by ``python -m tritonix_amd.build`` and is
+loaded from the package directory.  There is no fallback: if it is missing,
+every entry point raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+from tritonix_amd.testing import LDS_LIMIT_BYTES, OutOfResources
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtritonix_hip.so")
+
+# enum tnx_dtype
+F16, BF16, I8, I32, F32 = 0, 1, 2, 3, 4
+# enum tnx_epilogue
+EPI_NONE, EPI_GLU_SILU, EPI_GLU_SIGMOID, EPI_GLU_IDENTITY = 0, 1, 2, 3
+# enum tnx_status
+OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP = 0, 1, 2, 3, 4, 5
+
+EXPORTS = ("tnx_gemm", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
+           "tnx_gemm_default_config", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
+           "tnx_last_hip_error", "tnx_version")
+
+
+class GemmArgs(ctypes.Structure):
+    """struct tnx_gemm_args"""
+    _fields_ = [
+        ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p),
+        ("m", ctypes.c_int64), ("n", ctypes.c_int64), ("k", ctypes.c_int64),
+        ("stride_am", ctypes.c_int64), ("stride_ak", ctypes.c_int64),
+        ("stride_bk", ctypes.c_int64), ("stride_bn", ctypes.c_int64),
+        ("stride_cm", ctypes.c_int64), ("stride_cn", ctypes.c_int64),
+        ("in_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32),
+        ("block_m", ctypes.c_int32), ("block_n", ctypes.c_int32), ("block_k", ctypes.c_int32),
+        ("group_m", ctypes.c_int32), ("split_k", ctypes.c_int32),
+        ("num_stages", ctypes.c_int32), ("num_warps", ctypes.c_int32),
+        ("epilogue", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m tritonix_amd.build` "
+                           "(there is no non-HIP implementation to fall back to)")
+    lib = ctypes.CDLL(LIB_PATH)
+    p = ctypes.POINTER(GemmArgs)
+    lib.tnx_gemm.argtypes = [p]
+    lib.tnx_gemm.restype = ctypes.c_int
+    lib.tnx_gemm_workspace_bytes.argtypes = [p]
+    lib.tnx_gemm_workspace_bytes.restype = ctypes.c_size_t
+    lib.tnx_gemm_lds_bytes.argtypes = [p]
+    lib.tnx_gemm_lds_bytes.restype = ctypes.c_int64
+    lib.tnx_gemm_supported.argtypes = [p]
+    lib.tnx_gemm_supported.restype = ctypes.c_int
+    lib.tnx_gemm_default_config.argtypes = [p]
+    lib.tnx_gemm_default_config.restype = ctypes.c_int
+    lib.tnx_kernel_count.argtypes = []
+    lib.tnx_kernel_count.restype = ctypes.c_int
+    lib.tnx_kernel_name.argtypes = [ctypes.c_int]
+    lib.tnx_kernel_name.restype = ctypes.c_char_p
+    lib.tnx_strerror.argtypes = [ctypes.c_int]
+    lib.tnx_strerror.restype = ctypes.c_char_p
+    lib.tnx_last_hip_error.argtypes = []
+    lib.tnx_last_hip_error.restype = ctypes.c_int
+    lib.tnx_version.argtypes = []
+    lib.tnx_version.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def strerror(status: int) -> str:
+    return load().tnx_strerror(status).decode()
+
+
+def raise_for_status(status: int, args: GemmArgs) -> None:
+    """Map a tnx_status to the exception the tuner and the dispatcher expect."""
+    if status == OK:
+        return
+    lib = load()
+    if status == E_LDS:
+        raise OutOfResources(int(lib.tnx_gemm_lds_bytes(ctypes.byref(args))), LDS_LIMIT_BYTES, "shared memory")
+    if status == E_UNSUPPORTED:
+        raise ValueError(
+            f"{strerror(status)}: dtype={args.in_dtype} block=({args.block_m},{args.block_n},{args.block_k}) "
+            f"warps={args.num_warps} stages={args.num_stages} split_k={args.split_k} epilogue={args.epilogue}")
+    if status == E_HIP:
+        raise RuntimeError(f"{strerror(status)} (hipError_t {lib.tnx_last_hip_error()})")
+    if status == E_WORKSPACE:
+        raise RuntimeError(strerror(status))
+    raise ValueError(strerror(status))
+
+
+def kernel_names():
+    lib = load()
+    return [lib.tnx_kernel_name(i).decode() for i in range(lib.tnx_kernel_count())]

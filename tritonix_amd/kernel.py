@@ -1,0 +1,169 @@
+"""Launch objects that keep the reference's Triton calling convention over the HIP engine.
+
+A reference kernel is launched as ``kernel[grid](a, b, c, m, n, k, stride_am,
+stride_ak, stride_bk, stride_bn, stride_cm, stride_cn, block_m=..., block_n=...,
+block_k=..., group_m=..., [split_k=...,] num_stages=..., num_warps=...)``
+(tritonix/ops/matmul.py:222-236, :249-263; the GLU kernel adds ``use_tf32``
+and ``activation``, tritonix/ops/swiglu.py:24-43).  ``HipKernel`` accepts the
+same call, turns it into one ``tnx_gemm`` through the C ABI and launches on
+torch's current stream.  ``grid`` is accepted for compatibility; the engine
+derives its own 1-D grid from the shape and the tile.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Callable, Dict, List, Optional, Tuple
+
+from tritonix_amd import _C
+
+__all__ = ["HipKernel", "cdiv"]
+
+
+def cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+_POSITIONAL = ("a", "b", "c", "m", "n", "k", "stride_am", "stride_ak", "stride_bk", "stride_bn", "stride_cm",
+               "stride_cn")
+_ACTIVATIONS = {"silu": _C.EPI_GLU_SILU, "sigmoid": _C.EPI_GLU_SIGMOID}
+
+_workspaces: Dict[Tuple[int, int], object] = {}
+
+
+def _torch_dtype_code(dtype) -> int:
+    import torch
+
+    table = {torch.float16: _C.F16, torch.bfloat16: _C.BF16, torch.int8: _C.I8, torch.int32: _C.I32,
+             torch.float32: _C.F32}
+    if dtype not in table:
+        raise ValueError(f"dtype {dtype} has no HIP kernel (float16, bfloat16 and int8 inputs are built)")
+    return table[dtype]
+
+
+def out_dtype_for(dtype):
+    """Output dtype of the engine for an input dtype: 16-bit floats keep theirs, int8 accumulates to int32."""
+    import torch
+
+    return torch.int32 if dtype == torch.int8 else dtype
+
+
+def _workspace(device, stream_ptr: int, nbytes: int):
+    """Split-K scratch, one growing buffer per (device, stream); contents never need initialising."""
+    import torch
+
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+class _BoundLaunch:
+    def __init__(self, kernel: "HipKernel", grid):
+        self.kernel, self.grid = kernel, grid
+
+    def __call__(self, *args, **kwargs):
+        return self.kernel.run(*args, grid=self.grid, **kwargs)
+
+
+class HipKernel:
+    """One entry of the HIP engine behind the Triton launch protocol."""
+
+    def __init__(self, name: str, tile_params: List[str], glu: bool = False, doc: Optional[str] = None):
+        self.__name__ = name
+        self.__doc__ = doc
+        self.tile_params = list(tile_params)
+        self.glu = glu
+        self.arg_names = list(_POSITIONAL) + self.tile_params + (["use_tf32", "activation"] if glu else [])
+        self.pre_run_hooks: List[Callable] = []
+        self.specialize_keys: List[str] = []
+
+    def __getitem__(self, grid) -> _BoundLaunch:
+        return _BoundLaunch(self, grid)
+
+    def add_pre_run_hook(self, hook: Callable) -> None:
+        """``hook(*args, **kwargs)`` runs before every launch, as with a Triton ``JITFunction``."""
+        self.pre_run_hooks.append(hook)
+
+    # ------------------------------------------------------------------
+    def _bind(self, args, kwargs) -> dict:
+        if len(args) > len(self.arg_names):
+            raise TypeError(f"{self.__name__} takes at most {len(self.arg_names)} arguments, got {len(args)}")
+        bound = dict(zip(self.arg_names, args))
+        for k, v in kwargs.items():
+            if k not in self.arg_names:
+                raise TypeError(f"{self.__name__} got an unexpected keyword argument '{k}'")
+            if k in bound:
+                raise TypeError(f"{self.__name__} got multiple values for argument '{k}'")
+            bound[k] = v
+        missing = [n for n in list(_POSITIONAL) + self.tile_params if n not in bound]
+        if missing:
+            raise TypeError(f"{self.__name__} missing arguments: {', '.join(missing)}")
+        return bound
+
+    def make_args(self, bound: dict) -> _C.GemmArgs:
+        """Fill a ``tnx_gemm_args`` from a bound call (pointers from the tensors' ``data_ptr``)."""
+        a, b, c = bound["a"], bound["b"], bound["c"]
+        g = _C.GemmArgs()
+        g.a, g.b, g.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+        g.m, g.n, g.k = int(bound["m"]), int(bound["n"]), int(bound["k"])
+        g.stride_am, g.stride_ak = int(bound["stride_am"]), int(bound["stride_ak"])
+        g.stride_bk, g.stride_bn = int(bound["stride_bk"]), int(bound["stride_bn"])
+        g.stride_cm, g.stride_cn = int(bound["stride_cm"]), int(bound["stride_cn"])
+        g.in_dtype = _torch_dtype_code(a.dtype)
+        if b.dtype != a.dtype:
+            raise ValueError(f"a and b must share a dtype, got {a.dtype} and {b.dtype}")
+        g.out_dtype = _torch_dtype_code(c.dtype)
+        g.block_m, g.block_n, g.block_k = int(bound["block_m"]), int(bound["block_n"]), int(bound["block_k"])
+        g.group_m = int(bound["group_m"])
+        g.split_k = int(bound.get("split_k", 1))
+        g.num_stages, g.num_warps = int(bound["num_stages"]), int(bound["num_warps"])
+        if self.glu:
+            # "silu" and "sigmoid" gate explicitly; like the reference kernel, any other
+            # value leaves the gate un-activated (tritonix/ops/swiglu.py:100-102)
+            g.epilogue = _ACTIVATIONS.get(bound.get("activation", "silu"), _C.EPI_GLU_IDENTITY)
+        else:
+            g.epilogue = _C.EPI_NONE
+        return g
+
+    def run(self, *args, grid=None, **kwargs):
+        import torch
+
+        bound = self._bind(args, kwargs)
+        a, b, c = bound["a"], bound["b"], bound["c"]
+        for name, t in (("a", a), ("b", b), ("c", c)):
+            if not isinstance(t, torch.Tensor) or not t.is_cuda:
+                raise ValueError(f"{self.__name__}: '{name}' must be a tensor on a HIP device")
+        if not (a.device == b.device == c.device):
+            raise ValueError(f"{self.__name__}: a, b and c must live on one device")
+        if grid is not None and not callable(grid):
+            if not all(isinstance(g, int) and g >= 0 for g in tuple(grid)):
+                raise ValueError(f"{self.__name__}: grid must be a tuple of non-negative ints, got {grid!r}")
+        for hook in self.pre_run_hooks:
+            hook(*args, **kwargs)
+
+        lib = _C.load()
+        g = self.make_args(bound)
+        with torch.cuda.device(a.device):
+            stream = torch.cuda.current_stream(a.device).cuda_stream
+            g.stream = stream
+            if g.split_k > 1:
+                need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
+                if need:
+                    ws = _workspace(a.device, stream, need)
+                    g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
+            status = lib.tnx_gemm(ctypes.byref(g))
+        _C.raise_for_status(status, g)
+        return None
+
+    # host-only helpers -------------------------------------------------
+    def lds_bytes(self, in_dtype_code: int, block_m: int, block_n: int, block_k: int, num_stages: int) -> int:
+        """LDS bytes per workgroup of a tile config (no GPU needed)."""
+        g = _C.GemmArgs()
+        g.in_dtype = in_dtype_code
+        g.block_m, g.block_n, g.block_k, g.num_stages = block_m, block_n, block_k, num_stages
+        return int(_C.load().tnx_gemm_lds_bytes(ctypes.byref(g)))
+
+    def __repr__(self):
+        return f"<HipKernel {self.__name__}>"

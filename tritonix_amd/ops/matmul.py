@@ -1,0 +1,195 @@
+"""Dense GEMM ops: ``matmul`` (dispatcher), ``triton_matmul`` (tuned tiled GEMM), ``matmul_splitk``.
+
+Public surface and launch flow follow tritonix/ops/matmul.py of the reference:
+the ``@tunable`` kernels ``matmul_kernel`` (:30-108) and ``gemm_splitk_kernel``
+(:133-202), the host launchers ``_launch_matmul`` (:217-237) and
+``_launch_splitk`` (:240-264), the per-shape config memo and ``triton_matmul``
+/ ``matmul_splitk`` (:267-288) and the dispatcher instance ``matmul``
+(:291-293).  The kernels behind them are the gfx950 HIP tile kernels of
+libtritonix_hip.so; ``torch.matmul`` stays registered as the ``"pytorch"``
+backend and serves as the correctness oracle, exactly as in the reference.
+
+Deliberate differences:
+  * tile spaces are the ones that exist as HIP kernels (64..256 tiles, 2..4
+    LDS stages); a combination that is not built raises ``ValueError`` and the
+    tuner skips it, one that exceeds 160 KiB of LDS raises ``OutOfResources``
+    before any launch and the trie prunes above it;
+  * the config memo is keyed by dtype as well as (m, n, k), because one
+    process now runs f16, bf16 and int8 problems;
+  * int8 inputs give an int32 result;
+  * split-K sums fp32 partials from a workspace and rounds once, where the
+    reference rounds each partial to the output dtype and adds atomically
+    (tritonix/ops/matmul.py:195-202); the ``_zero_output`` hook is gone with it.
+"""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from tritonix_amd.autotune import Choice, PowerOfTwo, Range, tunable
+from tritonix_amd.dispatcher import dynamic_dispatch
+from tritonix_amd.kernel import HipKernel, cdiv, out_dtype_for
+
+__all__ = ["matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel", "gemm_splitk_kernel",
+           "swizzle2d", "grouped_launch", "TUNE_OPTIONS"]
+
+# keyword arguments handed to ``.tune`` on a config-memo miss (tests shrink the time budgets)
+TUNE_OPTIONS = {"warmup": 25, "rep": 100}
+
+_TILE = ["block_m", "block_n", "block_k", "group_m", "num_stages", "num_warps"]
+
+matmul_kernel = tunable(
+    keys=["m", "n", "k"],
+    space={
+        "block_m": PowerOfTwo(64, 256),
+        "block_n": PowerOfTwo(64, 256),
+        "block_k": PowerOfTwo(32, 128),
+        "group_m": Choice([4, 8]),
+        "num_stages": Range(2, 4),
+        "num_warps": Choice([4, 8]),
+    },
+    memory_params={"block_m", "block_n", "block_k", "num_stages"},
+)(HipKernel("matmul_kernel", _TILE, doc="C = A x B. A has shape (M, K), B has shape (K, N) and C has shape (M, N)"))
+
+gemm_splitk_kernel = tunable(
+    keys=["m", "n", "k"],
+    space={
+        "block_m": PowerOfTwo(64, 128),
+        "block_n": PowerOfTwo(64, 256),
+        "block_k": PowerOfTwo(32, 128),
+        "group_m": Choice([4, 8]),
+        "split_k": PowerOfTwo(2, 16),
+        "num_stages": Range(2, 4),
+        "num_warps": Choice([4, 8]),
+    },
+    memory_params={"block_m", "block_n", "block_k", "num_stages"},
+)(HipKernel("gemm_splitk_kernel", ["block_m", "block_n", "block_k", "group_m", "split_k", "num_stages", "num_warps"],
+            doc="C = A x B with K cut into split_k slices; fp32 partials, one rounding"))
+
+
+def swizzle2d(i, j, size_i, size_j, size_g):
+    """Tile-id remap the kernels apply: rows of tiles are walked in groups of ``size_g``, column-major inside a group.
+
+    Same mapping as ``tl.swizzle2d`` (called at tritonix/ops/matmul.py:70); host-side copy for tests and tooling.
+    """
+    ij = i * size_j + j
+    per_group = size_g * size_j
+    first_row = (ij // per_group) * size_g
+    rows = min(size_i - first_row, size_g)
+    r = ij % per_group
+    return first_row + r % rows, r // rows
+
+
+def grouped_launch(pid, m, n, block_m, block_n, group_m):
+    """1-D program id -> (pid_m, pid_n) in grouped order.
+
+    Same intent as the reference's unused helper (tritonix/ops/matmul.py:111-130) but computed with the
+    ``swizzle2d`` formula, which stays a bijection when the last group of tile rows is ragged.
+    """
+    grid_m, grid_n = cdiv(m, block_m), cdiv(n, block_n)
+    return swizzle2d(pid // grid_n, pid % grid_n, grid_m, grid_n, group_m)
+
+
+def _check_2d(a, b):
+    if a.dim() != 2 or b.dim() != 2:
+        raise ValueError(f"matmul expects 2-D tensors, got {tuple(a.shape)} and {tuple(b.shape)}")
+    if a.shape[1] != b.shape[0]:
+        raise ValueError(f"inner dimensions differ: {tuple(a.shape)} @ {tuple(b.shape)}")
+
+
+def _launch_matmul(a, b, cfg):
+    m, k = a.shape
+    _, n = b.shape
+    c = torch.empty((m, n), device=a.device, dtype=out_dtype_for(a.dtype))
+    grid = (cdiv(m, cfg["block_m"]), cdiv(n, cfg["block_n"]))
+    matmul_kernel[grid](a, b, c, m, n, k, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                        **cfg)
+    return c
+
+
+def _launch_splitk(a, b, cfg):
+    m, k = a.shape
+    _, n = b.shape
+    # no zero fill: the kernel owns its workspace and writes every element of c
+    c = torch.empty((m, n), device=a.device, dtype=out_dtype_for(a.dtype))
+    grid = (cdiv(m, cfg["block_m"]), cdiv(n, cfg["block_n"]), cfg["split_k"])
+    gemm_splitk_kernel[grid](a, b, c, m, n, k, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0),
+                             c.stride(1), **cfg)
+    return c
+
+
+_matmul_cfg = {}
+_splitk_cfg = {}
+
+
+def default_config(a, b, split=False):
+    """The engine's built-in tile choice for this problem (used when tuning is switched off)."""
+    import ctypes
+
+    from tritonix_amd import _C
+    from tritonix_amd.kernel import _torch_dtype_code
+
+    g = _C.GemmArgs()
+    g.m, g.k = a.shape
+    g.n = b.shape[1]
+    g.in_dtype = _torch_dtype_code(a.dtype)
+    _C.load().tnx_gemm_default_config(ctypes.byref(g))
+    cfg = {"block_m": g.block_m, "block_n": g.block_n, "block_k": g.block_k, "group_m": g.group_m,
+           "num_stages": g.num_stages, "num_warps": g.num_warps}
+    if split:
+        cfg["split_k"] = max(2, g.split_k)
+    return cfg
+
+
+def _autotune_enabled() -> bool:
+    return os.environ.get("TRITONIX_AUTOTUNE", "1") not in ("0", "false", "False")
+
+
+def triton_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """C = A @ B on the HIP tile kernel, tile config tuned once per (m, n, k, dtype).
+
+    Keeps the reference's name: callers and the ``"triton"`` backend label of
+    ``matmul`` refer to it.  ``hip_matmul`` is the same function.
+    """
+    _check_2d(a, b)
+    m, k = a.shape
+    _, n = b.shape
+    key = (m, n, k, a.dtype)
+    if key not in _matmul_cfg:
+        if _autotune_enabled():
+            cfg = matmul_kernel.tune(lambda cfg: _launch_matmul(a, b, cfg), **TUNE_OPTIONS)
+            if cfg is None:
+                raise RuntimeError(f"no HIP tile kernel accepts {tuple(a.shape)} @ {tuple(b.shape)} {a.dtype}")
+            _matmul_cfg[key] = cfg
+        else:
+            _matmul_cfg[key] = default_config(a, b)
+    return _launch_matmul(a, b, _matmul_cfg[key])
+
+
+hip_matmul = triton_matmul
+
+
+def matmul_splitk(a: torch.Tensor, b: torch.Tensor, split_k: int = 4) -> torch.Tensor:
+    """Split-K GEMM for skinny shapes.
+
+    As in the reference (tritonix/ops/matmul.py:280-288) ``split_k`` only keys
+    the config memo; the split factor launched is the one the tuner picked.
+    """
+    _check_2d(a, b)
+    m, k = a.shape
+    _, n = b.shape
+    key = (m, n, k, split_k, a.dtype)
+    if key not in _splitk_cfg:
+        if _autotune_enabled():
+            cfg = gemm_splitk_kernel.tune(lambda cfg: _launch_splitk(a, b, cfg), **TUNE_OPTIONS)
+            if cfg is None:
+                raise RuntimeError(f"no HIP split-K kernel accepts {tuple(a.shape)} @ {tuple(b.shape)} {a.dtype}")
+            _splitk_cfg[key] = cfg
+        else:
+            _splitk_cfg[key] = default_config(a, b, split=True)
+    return _launch_splitk(a, b, _splitk_cfg[key])
+
+
+matmul = dynamic_dispatch({"triton": triton_matmul, "pytorch": torch.matmul}, key=["a", "b"])
+matmul.alias("hip", "triton")
