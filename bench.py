@@ -84,6 +84,14 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
 
+    # one plain device copy of known size (2^28 bytes read, 2^28 written): under `rocprofv3 --pmc
+    # FETCH_SIZE` / `WRITE_SIZE` it is the dispatch the GEMM's counter readings are scaled by
+    cal_src = torch.empty(1 << 28, dtype=torch.uint8, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     # ---- headline: C2 --------------------------------------------------------------
     a_cpu, b_cpu = oracle.make_inputs("C2")
     a, b = a_cpu.to(dev), b_cpu.to(dev)

@@ -155,22 +155,22 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
 extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   if (!a) return TNX_E_INVALID;
   const int es = elem_size(a->in_dtype);
+  const int bk = es == 1 ? 128 : 64;   // 128 bytes of K per LDS row for either element size
   a->group_m = 8;
   a->split_k = 1;
-  a->num_warps = 4;
   if (a->m <= 64) {
-    // skinny: stream B, split K to fill the chip
-    a->block_m = 64; a->block_n = 128; a->block_k = 64 / es * 2 > 64 ? 128 : 64; a->num_stages = 3;
-    a->block_k = es == 1 ? 128 : 64;
+    // skinny: B is streamed once, K is split until the grid covers the chip a few times over
+    a->block_m = 64; a->block_n = 128; a->block_k = bk; a->num_stages = 3; a->num_warps = 4;
     int64_t tiles = (a->n + a->block_n - 1) / a->block_n;
     int64_t kt = (a->k + a->block_k - 1) / a->block_k;
     int s = 1;
     while (tiles * s < 512 && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
     a->split_k = s;
   } else if (a->m >= 2048 && a->n >= 2048) {
-    a->block_m = 256; a->block_n = 256; a->block_k = es == 1 ? 128 : 64; a->num_stages = 2;
+    // two waves per SIMD fill each other's issue gaps on the 256x256 tile
+    a->block_m = 256; a->block_n = 256; a->block_k = bk; a->num_stages = 2; a->num_warps = 8;
   } else {
-    a->block_m = 128; a->block_n = 128; a->block_k = es == 1 ? 128 : 64; a->num_stages = 3;
+    a->block_m = 128; a->block_n = 128; a->block_k = bk; a->num_stages = 3; a->num_warps = 4;
   }
   return TNX_OK;
 }

@@ -51,7 +51,7 @@ struct GemmParams {
   int ktiles_per_split;   // K slabs handled by one split
   int epilogue;
   int out_dtype;
-  bool c_vec_ok;          // C allows 4-element vector stores along n (stride_cn == 1, aligned)
+  bool c_vec_ok;          // C takes 16-byte stores along n (stride_cn == 1, 16-byte aligned rows)
 };
 
 // ---------------------------------------------------------------------------
@@ -133,6 +133,12 @@ __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint3
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
                : "memory");
+}
+
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+  uint64_t v = (uint64_t)(uintptr_t)p;
+  uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
 template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
@@ -219,7 +225,7 @@ struct TileCfg {
 };
 
 // ---------------------------------------------------------------------------
-// output conversion and the store of one accumulator tile set
+// output conversion and the store of a wave's accumulators
 // ---------------------------------------------------------------------------
 struct OutBF16 { typedef uint16_t raw; static __device__ __forceinline__ raw cvt(float v) { return f32_to_bf16(v); } };
 struct OutF16 {
@@ -235,64 +241,94 @@ template <class O, class S> struct Cvt { typedef typename O::raw raw; static __d
 template <> struct Cvt<float, float> { typedef float raw; static __device__ __forceinline__ float run(float v) { return v; } };
 template <> struct Cvt<int, int> { typedef int raw; static __device__ __forceinline__ int run(int v) { return v; } };
 
-// GLU != 0: columns (2c, 2c+1) hold (gate, linear); output column c.
+// Bytes of LDS one wave needs to transpose one row-block (MI rows) of its
+// output through LDS; rows are padded by 16 bytes to spread the banks.
+template <class C, int OES> struct EpiStage {
+  static constexpr int PITCH = C::WTN * OES + 16;
+  static constexpr int WAVE_BYTES = C::MI * PITCH;
+  static constexpr int BYTES = C::NW * WAVE_BYTES;
+};
+
+// The MFMA result is C^T: lane l owns output row m = l % MI and, per group of
+// four accumulator registers, four consecutive columns n.  Each wave writes
+// one row-block at a time into its private LDS strip ([MI rows][wave-tile
+// columns], output dtype, gating already applied), reads it back row-major
+// and stores 16 bytes per lane, so every row of C receives full contiguous
+// runs instead of 8-byte fragments.  GLU != 0: columns (2c, 2c+1) hold
+// (gate, linear); output column c.
 template <class T, class C, class O, int GLU, class ACC>
-__device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, int64_t gm_base, int64_t gn_base,
-                                               int64_t m, int64_t n, int64_t scm, int64_t scn, bool vec_ok, int epi) {
+__device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t lds_strip, int lane,
+                                               int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
+                                               int64_t scn, bool vec_ok, int epi) {
   typedef typename T::acc_s acc_s;
   typedef Cvt<O, acc_s> CV;
   typedef typename CV::raw raw;
   constexpr int MI = C::MI;
-  constexpr int NGRP = C::ACC_N / 4;        // groups of four consecutive columns per accumulator tile
+  constexpr int OES = sizeof(raw);
+  constexpr int NGRP = C::ACC_N / 4;                    // groups of four consecutive columns per accumulator tile
+  constexpr int WCOLS = GLU ? C::WTN / 2 : C::WTN;      // output columns of the wave tile
+  constexpr int PITCH = C::WTN * OES + 16;              // strip pitch (sized for the non-GLU case)
+  constexpr int VEC = 16 / OES;                         // elements per 16-byte store
+  constexpr int CPRW = WCOLS / VEC;                     // 16-byte chunks per strip row
+  constexpr int ITERS = (MI * CPRW + 63) / 64;
+  static_assert(WCOLS % VEC == 0, "wave tile too narrow for 16-byte stores");
   raw* cp = (raw*)cbase;
+  const int wrow = lane % MI, wcol = (lane / MI) * 4;
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
-    const int64_t gm = gm_base + i * MI;
-    if (gm >= m) continue;
+    // ---- registers -> strip
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
 #pragma unroll
       for (int g = 0; g < NGRP; ++g) {
-        const int64_t gn = gn_base + j * MI + g * 8;
+        const int col = j * MI + g * 8 + wcol;          // column inside the wave tile (interleaved width)
         acc_s v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
-        if (GLU) {
-          const int64_t nh = n >> 1, gc = gn >> 1;
+        if constexpr (GLU) {
           raw z0 = CV::run((acc_s)(glu_gate((float)v0, epi) * (float)v1));
           raw z1 = CV::run((acc_s)(glu_gate((float)v2, epi) * (float)v3));
-          raw* dst = cp + gm * scm + gc * scn;
-          if (vec_ok && gc + 1 < nh) {
-            if constexpr (sizeof(raw) == 2) *(uint32_t*)dst = (uint32_t)z0 | ((uint32_t)z1 << 16);
-            else { dst[0] = z0; dst[1] = z1; }
-          } else {
-            if (gc < nh) dst[0] = z0;
-            if (gc + 1 < nh) dst[scn] = z1;
-          }
+          const uint32_t dst = lds_strip + wrow * PITCH + (col >> 1) * OES;
+          if constexpr (OES == 2) *TNX_LDS(uint32_t, dst) = (uint32_t)z0 | ((uint32_t)z1 << 16);
+          else *TNX_LDS(i32x2, dst) = i32x2{__builtin_bit_cast(int, z0), __builtin_bit_cast(int, z1)};
         } else {
           raw r0 = CV::run(v0), r1 = CV::run(v1), r2 = CV::run(v2), r3 = CV::run(v3);
-          raw* dst = cp + gm * scm + gn * scn;
-          if (vec_ok && gn + 3 < n) {
-            if constexpr (sizeof(raw) == 2) {
-              uint2 pk;
-              pk.x = (uint32_t)r0 | ((uint32_t)r1 << 16);
-              pk.y = (uint32_t)r2 | ((uint32_t)r3 << 16);
-              *(uint2*)dst = pk;
-            } else {
-              uint4 pk;
-              pk.x = __builtin_bit_cast(uint32_t, r0); pk.y = __builtin_bit_cast(uint32_t, r1);
-              pk.z = __builtin_bit_cast(uint32_t, r2); pk.w = __builtin_bit_cast(uint32_t, r3);
-              *(uint4*)dst = pk;
-            }
-          } else {
-            if (gn < n) dst[0] = r0;
-            if (gn + 1 < n) dst[scn] = r1;
-            if (gn + 2 < n) dst[2 * scn] = r2;
-            if (gn + 3 < n) dst[3 * scn] = r3;
-          }
+          const uint32_t dst = lds_strip + wrow * PITCH + col * OES;
+          if constexpr (OES == 2)
+            *TNX_LDS(i32x2, dst) = i32x2{(int)((uint32_t)r0 | ((uint32_t)r1 << 16)), (int)((uint32_t)r2 | ((uint32_t)r3 << 16))};
+          else
+            *TNX_LDS(i32x4, dst) = i32x4{__builtin_bit_cast(int, r0), __builtin_bit_cast(int, r1),
+                                         __builtin_bit_cast(int, r2), __builtin_bit_cast(int, r3)};
         }
       }
     }
+    // the strip is private to this wave: its own LDS writes are ordered before its reads
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    // ---- strip -> global, row-major 16-byte chunks
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int q = it * 64 + lane;
+      const int row = q / CPRW, cc = q % CPRW;
+      if (MI * CPRW % 64 != 0 && row >= MI) continue;
+      const int64_t gm = gm0 + i * MI + row;
+      const int64_t gc = gc0 + cc * VEC;
+      i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + cc * 16);
+      if (gm >= m) continue;
+      raw* dst = cp + gm * scm + gc * scn;
+      if (vec_ok && gc + VEC <= ncols) {
+        *(i32x4*)dst = v;
+      } else {
+        raw e[VEC];
+        __builtin_memcpy(e, &v, 16);
+#pragma unroll
+        for (int x = 0; x < VEC; ++x)
+          if (gc + x < ncols) dst[x * scn] = e[x];
+      }
+    }
+    // the next row-block overwrites the strip: wait for the reads above
+    __builtin_amdgcn_s_waitcnt(0xC07F);
   }
 }
+
+template <bool B> struct BoolTag { static constexpr bool value = B; };
 
 // ---------------------------------------------------------------------------
 // the kernel
@@ -305,7 +341,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
 
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[C::LDS_BYTES];
+  constexpr int SMEM_BYTES = C::LDS_BYTES > EpiStage<C, 4>::BYTES ? C::LDS_BYTES : EpiStage<C, 4>::BYTES;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[SMEM_BYTES];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
 
   const int tid = threadIdx.x;
@@ -338,8 +375,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const uint8_t* b_sbase = p.b;
   if (FAST) {
     const int64_t lda = p.sam, ldb = p.sbk;
-    a_sbase = p.a + (m0 * lda + (int64_t)kt0 * BK) * ES;
-    b_sbase = p.b + ((int64_t)kt0 * BK * ldb + n0) * ES;
+    // wave-uniform by construction; say so, so both stay in SGPRs for the DMA's scalar base operand
+    a_sbase = uniform_ptr(p.a + (m0 * lda + (int64_t)kt0 * BK) * ES);
+    b_sbase = uniform_ptr(p.b + ((int64_t)kt0 * BK * ldb + n0) * ES);
     const int64_t mrem = p.m - 1 - m0;  // last valid row inside this tile
 #pragma unroll
     for (int q = 0; q < C::A_LPW; ++q) {
@@ -459,16 +497,36 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   };
 
   // ---- pipeline ----------------------------------------------------------
-  // Ring of STAGES slabs.  Inside the iteration of slab t the barrier sits
-  // before the last k step: by then every wave has read all of slab t, so its
-  // slot is handed to the DMA of slab t+STAGES, and slab t+1 is known to have
-  // landed, so its first fragments are fetched under the last k step's MFMAs.
-  // The K loop is cut in three (DMA still to issue / ring draining / final
-  // slab) so the accumulators flow through straight-line code.
+  // Ring of STAGES slabs, one workgroup barrier per slab.  barrier(t) sits
+  // before the last k step of slab t: every wave has then issued and received
+  // all its LDS reads of slab t, so the slot of slab t is handed to the DMA of
+  // slab t+STAGES, and slab t+1 is known to have landed, so its first
+  // fragments are fetched under the last k step's MFMAs.  A "period" is the
+  // code between barrier(t) and barrier(t+1): the last k step of slab t, then
+  // k steps 0..KSTEPS-2 of slab t+1.  The DMA ops of one refill are slotted
+  // behind the period's MFMAs at an even rate (a burst of them backs up the
+  // texture-address queue and stalls the wave); with only two slabs in the
+  // ring the refill is due at the very next barrier, so it is issued in the
+  // first k step of the period instead.  The K loop is cut in three (refills
+  // to issue / ring draining / final step) so the accumulators flow through
+  // straight-line code.
+  constexpr int PERIOD = C::KSTEPS * NMMA;                       // MFMA slots per period
+  constexpr int SPAN = (STAGES == 2 || !FAST) ? NMMA : PERIOD;   // slots the refill is spread over
+  constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
+  constexpr int NEXT0 = C::KSTEPS & 1;                           // set that receives step 0 of the next slab
 
-  // k steps 0 .. KSTEPS-2 of the slab at (sa, sb): multiply register set
-  // (ks & 1) while filling the other set with step ks+1
-  auto inner_steps = [&](uint32_t sa, uint32_t sb) {
+  // DMA ops due at period slot `slot` (compile-time after unrolling)
+  auto dma_slot = [&](int slot, uint32_t dst) {
+    if (slot < SPAN) {
+      const int lo = slot * C::LPW / SPAN, hi = (slot + 1) * C::LPW / SPAN;
+#pragma unroll
+      for (int q = lo; q < hi; ++q) dma_op(q, dst);
+    }
+  };
+  // k steps 0 .. KSTEPS-2 of the slab at (sa, sb): multiply register set (ks & 1) while filling
+  // the other set with step ks+1; WITH_DMA: keep issuing the refill into slot `dst`
+  auto inner_steps = [&](uint32_t sa, uint32_t sb, auto with_dma, uint32_t dst) {
+    constexpr bool WITH_DMA = decltype(with_dma)::value;
 #pragma unroll
     for (int ks = 0; ks + 1 < C::KSTEPS; ++ks) {
       int rd = 0;
@@ -478,14 +536,25 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
 #pragma unroll
         for (int q = 0; q < RPM; ++q)
           if (rd < NREAD) { read_one((ks + 1) & 1, rd, sa, sb, ks + 1); ++rd; }
+        if constexpr (WITH_DMA) dma_slot(NMMA + ks * NMMA + x, dst);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
-  constexpr int LAST = (C::KSTEPS - 1) & 1;   // register set holding the last k step
-  constexpr int NEXT0 = C::KSTEPS & 1;        // set that receives step 0 of the next slab
-  auto swap_sets = [&]() {                    // odd KSTEPS: the sets trade roles every slab
-    if (C::KSTEPS & 1) {
+  // last k step of the slab whose fragments sit in set LAST; prefetches step 0 of the slab at (sa1, sb1)
+  auto last_step = [&](uint32_t sa1, uint32_t sb1, auto with_dma, uint32_t dst) {
+    constexpr bool WITH_DMA = decltype(with_dma)::value;
+    int rd = 0;
+#pragma unroll
+    for (int x = 0; x < NMMA; ++x) {
+      mma_one(LAST, x);
+#pragma unroll
+      for (int q = 0; q < RPM; ++q)
+        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
+      if constexpr (WITH_DMA) dma_slot(x, dst);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (C::KSTEPS & 1) {   // odd KSTEPS: the two register sets trade roles every slab
 #pragma unroll
       for (int i = 0; i < TM; ++i) { i32x4 tmp = fa[0][i]; fa[0][i] = fa[1][i]; fa[1][i] = tmp; }
 #pragma unroll
@@ -494,6 +563,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         for (int h = 0; h < 2; ++h) { i32x2 tmp = fb[0][j][h]; fb[0][j][h] = fb[1][j][h]; fb[1][j][h] = tmp; }
     }
   };
+  typedef BoolTag<true> Yes;
+  typedef BoolTag<false> No;
 
   if (KT > 0) {
 #pragma unroll
@@ -513,79 +584,58 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
 #pragma unroll
     for (int r = 0; r < NREAD; ++r) read_one(0, r, sa, sb, 0);
+    inner_steps(sa, sb, No{}, 0u);
   }
 
   int t = 0;
-  // (1) slabs whose slot is refilled by the DMA of slab t+STAGES
+  // (1) periods that issue the refill of slab t+STAGES into the slot of slab t
   for (; t + STAGES < KT; ++t) {
-    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
-    inner_steps(sa, sb);
     __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, sa);
+    const uint32_t dst = stage_of(t);
+    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
-    int rd = 0, dq = 0;
-#pragma unroll
-    for (int x = 0; x < NMMA; ++x) {
-      mma_one(LAST, x);
-#pragma unroll
-      for (int q = 0; q < RPM; ++q)
-        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
-      if constexpr (FAST) {
-#pragma unroll
-        for (int q = 0; q < DPM; ++q)
-          if (dq < C::LPW) { dma_op(dq, sa); ++dq; }
-      }
-      __builtin_amdgcn_sched_barrier(0);
+    if constexpr (FAST) {
+      last_step(sa1, sb1, Yes{}, dst);
+      inner_steps(sa1, sb1, Yes{}, dst);
+      dma_advance();
+    } else {
+      last_step(sa1, sb1, No{}, 0u);
+      inner_steps(sa1, sb1, No{}, 0u);
     }
-    if constexpr (FAST) dma_advance();
-    swap_sets();
   }
   // (2) ring draining: nothing left to issue
   for (; t + 1 < KT; ++t) {
-    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
-    inner_steps(sa, sb);
     __builtin_amdgcn_s_waitcnt(0x0070);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
-    int rd = 0;
-#pragma unroll
-    for (int x = 0; x < NMMA; ++x) {
-      mma_one(LAST, x);
-#pragma unroll
-      for (int q = 0; q < RPM; ++q)
-        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    swap_sets();
+    last_step(sa1, sb1, No{}, 0u);
+    inner_steps(sa1, sb1, No{}, 0u);
   }
-  // (3) final slab
+  // (3) last k step of the final slab
   if (KT > 0) {
-    const uint32_t sa = stage_of(t), sb = sa + C::A_BYTES;
-    inner_steps(sa, sb);
 #pragma unroll
     for (int x = 0; x < NMMA; ++x) mma_one(LAST, x);
   }
 
   // ---- epilogue ------------------------------------------------------------
-  // The MFMA was issued with the B fragment as its row operand, so the tile it
-  // returns is C^T: lane l owns output row m = l % MI and, per group of four
-  // accumulator registers, four consecutive columns n.  Four columns make one
-  // 8-byte (16-bit out) or 16-byte (32-bit out) store, and a gate/linear pair
-  // of the GLU epilogue sits inside one lane.
-  const int64_t gm_base = m0 + wy * C::WTM + (lane % MI);
-  const int64_t gn_base = n0 + wx * C::WTN + (lane / MI) * 4;
+  // every wave is done with the slabs before the LDS is reused for the output strips
+  __syncthreads();
+  const int64_t gm0 = m0 + wy * C::WTM;
+  const int64_t gn0 = n0 + wx * C::WTN;
   if (p.split_k > 1) {
     acc_s* ws = (acc_s*)p.ws + (int64_t)split * p.m * p.n;
-    epilogue_store<T, C, acc_s, EPI_NONE>(acc, (uint8_t*)ws, gm_base, gn_base, p.m, p.n, p.n, 1, (p.n & 3) == 0, 0);
-  } else if (p.epilogue == EPI_NONE) {
-    epilogue_store<T, C, typename OutOf<T>::type, EPI_NONE>(acc, p.c, gm_base, gn_base, p.m, p.n, p.scm, p.scn,
-                                                            p.c_vec_ok, 0);
+    const uint32_t strip = lds0 + wave * EpiStage<C, 4>::WAVE_BYTES;
+    epilogue_store<T, C, acc_s, 0>(acc, (uint8_t*)ws, strip, lane, gm0, gn0, p.m, p.n, p.n, 1, (p.n & 3) == 0, 0);
   } else {
-    epilogue_store<T, C, typename OutOf<T>::type, 1>(acc, p.c, gm_base, gn_base, p.m, p.n, p.scm, p.scn, p.c_vec_ok,
-                                                     p.epilogue);
+    typedef typename OutOf<T>::type O;
+    const uint32_t strip = lds0 + wave * EpiStage<C, sizeof(typename Cvt<O, acc_s>::raw)>::WAVE_BYTES;
+    if (p.epilogue == EPI_NONE)
+      epilogue_store<T, C, O, 0>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+    else
+      epilogue_store<T, C, O, 1>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
   }
 }
 
