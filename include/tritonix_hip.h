@@ -79,7 +79,7 @@ typedef struct tnx_gemm_args {
   int32_t num_stages; /* LDS ring depth of the global->LDS pipeline              */
   int32_t num_warps;  /* wavefronts (64 lanes) per workgroup: 4 or 8             */
   int32_t epilogue;   /* tnx_epilogue                                            */
-  void* workspace;    /* device scratch for split_k > 1, else may be NULL        */
+  void* workspace;    /* device scratch for split_k > 1 (see tnx_gemm_workspace_bytes) */
   size_t workspace_bytes;
   void* stream;       /* hipStream_t; NULL = the null stream                     */
 } tnx_gemm_args;
@@ -88,8 +88,14 @@ typedef struct tnx_gemm_args {
 int tnx_gemm(const tnx_gemm_args* args);
 
 /* Bytes of device scratch tnx_gemm needs for these args (0 when split_k <= 1).
- * The contents need no initialisation: the kernels own it (this replaces the
- * reference's `_zero_output` hook, tritonix/ops/matmul.py:205-210). */
+ * The workspace must be 256-byte aligned.  Its first TNX_WS_COUNTER_BYTES hold
+ * per-tile arrival counters: they must be zero before the first launch that
+ * uses the workspace, and every launch leaves them zero again, so one
+ * zero-fill at allocation is enough (calls sharing a workspace must be
+ * ordered on one stream).  The rest needs no initialisation.  C itself is
+ * never pre-zeroed: this replaces the reference's `_zero_output` hook
+ * (tritonix/ops/matmul.py:205-210). */
+#define TNX_WS_COUNTER_BYTES 65536
 size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* args);
 
 /* LDS bytes per workgroup the tile config in `args` would use.  Pure host

@@ -95,7 +95,7 @@ def test_ragged_layouts_need_a_generic_kernel():
 def test_workspace_bytes_and_default_config():
     lib = _C.load()
     assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args())) == 0
-    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=16, n=4096, k=14336, split_k=8))) == 8 * 16 * 4096 * 4
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=16, n=4096, k=14336, split_k=8))) == 65536 + 8 * 16 * 4096 * 4
     g = args(m=8192, n=8192, k=8192)
     assert lib.tnx_gemm_default_config(ctypes.byref(g)) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK

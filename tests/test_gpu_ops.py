@@ -128,3 +128,42 @@ def test_do_bench_returns_sane_numbers(device):
     assert 0 < tflops < 1e4
     q = do_bench(lambda: torch.matmul(a, a), warmup=2, rep=10, quantiles=[0.5, 0.2, 0.8])
     assert len(q) == 3 and q[1] <= q[0] <= q[2]
+
+
+def test_prepared_launch_repeats_one_c_abi_call(device):
+    a, b = oracle.make_inputs("C3", scale_down=4)
+    ad, bd = a.to(device), b.to(device)
+    m, k = ad.shape
+    n = bd.shape[1]
+    c = torch.zeros((m, n), device=device, dtype=torch.bfloat16)
+    cfg = mm.default_config(ad, bd, split=True)
+    launch = tritonix_amd.gemm_splitk_kernel.prepare(ad, bd, c, m, n, k, k, 1, n, 1, n, 1, **cfg)
+    launch()
+    first = c.clone()
+    for _ in range(5):                     # the counters of the workspace are re-armed by every launch
+        c.zero_()
+        launch()
+    assert torch.equal(c, first)
+    assert oracle.within_tolerance(c, oracle.reference_matmul(a, b))[0]
+    with pytest.raises(ValueError):
+        tritonix_amd.matmul_kernel.prepare(ad, bd, c, m, n, k, k, 1, n, 1, n, 1, block_m=96, block_n=128, block_k=64,
+                                           group_m=8, num_stages=2, num_warps=4)
+
+
+@pytest.mark.parametrize("shape", [(1024, 768, 512), (300, 200, 128), (4096, 4096, 1024), (64, 8192, 2048)])
+def test_default_configs_are_valid_and_correct(device, shape):
+    m, n, k = shape
+    g = torch.Generator("cpu").manual_seed(m + n)
+    for dt in (torch.float16, torch.int8):
+        if dt == torch.int8:
+            a = torch.randint(-127, 128, (m, k), generator=g, dtype=dt)
+            b = torch.randint(-127, 128, (k, n), generator=g, dtype=dt)
+        else:
+            a, b = torch.randn(m, k, generator=g).to(dt), torch.randn(k, n, generator=g).to(dt)
+        cfg = mm.default_config(a, b)
+        out = mm._launch_matmul(a.to(device), b.to(device), cfg)
+        ref = oracle.reference_matmul(a, b)
+        if dt == torch.int8:
+            assert torch.equal(out.cpu(), ref)
+        else:
+            assert oracle.within_tolerance(out, ref)[0]

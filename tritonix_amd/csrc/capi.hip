@@ -75,7 +75,7 @@ extern "C" int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* a) {
 
 extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
   if (!a || a->split_k <= 1 || a->m <= 0 || a->n <= 0) return 0;
-  return (size_t)a->split_k * (size_t)a->m * (size_t)a->n * 4;
+  return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)a->m * (size_t)a->n * 4;
 }
 
 static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs) {
@@ -91,6 +91,7 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   if (!f && !e->generic) return TNX_E_UNSUPPORTED;
   int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
   if (tiles * a->split_k > 0x7fffffffll) return TNX_E_UNSUPPORTED;
+  if (a->split_k > 1 && tiles > WS_MAX_TILES) return TNX_E_UNSUPPORTED;  // one arrival counter per tile
   if (out) *out = e;
   if (fast) *fast = f;
   return TNX_OK;
@@ -108,7 +109,8 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
     if (!a->c || (a->k > 0 && (!a->a || !a->b))) return TNX_E_INVALID;
   }
   if (a->m == 0 || a->n == 0) return TNX_OK;
-  if (a->split_k > 1 && (!a->workspace || a->workspace_bytes < tnx_gemm_workspace_bytes(a))) return TNX_E_WORKSPACE;
+  if (a->split_k > 1 && (!a->workspace || a->workspace_bytes < tnx_gemm_workspace_bytes(a) || ((uintptr_t)a->workspace & 255)))
+    return TNX_E_WORKSPACE;
 
   const int es_out = elem_size(a->out_dtype);
   GemmParams p;
@@ -129,26 +131,13 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.ktiles_per_split = (kt_total + a->split_k - 1) / a->split_k;
   p.epilogue = a->epilogue;
   p.out_dtype = a->out_dtype;
-  p.c_vec_ok = a->stride_cn == 1 && (a->stride_cm % 4) == 0 && (((uintptr_t)a->c) % (4 * es_out)) == 0;
+  p.c_vec_ok = a->stride_cn == 1 && ((a->stride_cm * es_out) % 16) == 0 && (((uintptr_t)a->c) % 16) == 0;
 
   hipStream_t stream = (hipStream_t)a->stream;
   unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * a->split_k);
   hipError_t err = (fast ? e->fast : e->generic)(p, grid, stream);
   if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
 
-  if (a->split_k > 1) {
-    int64_t ncols = a->epilogue == TNX_EPI_NONE ? a->n : a->n / 2;
-    int64_t total = a->m * ncols;
-    unsigned rgrid = (unsigned)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
-    if (a->in_dtype == TNX_I8)
-      hipLaunchKernelGGL((splitk_reduce_kernel<int>), dim3(rgrid), dim3(256), 0, stream, (const int*)p.ws, p.c, p.m, p.n,
-                         p.scm, p.scn, p.split_k, p.epilogue, p.out_dtype);
-    else
-      hipLaunchKernelGGL((splitk_reduce_kernel<float>), dim3(rgrid), dim3(256), 0, stream, (const float*)p.ws, p.c, p.m,
-                         p.n, p.scm, p.scn, p.split_k, p.epilogue, p.out_dtype);
-    err = hipGetLastError();
-    if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
-  }
   return TNX_OK;
 }
 
@@ -156,21 +145,42 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   if (!a) return TNX_E_INVALID;
   const int es = elem_size(a->in_dtype);
   const int bk = es == 1 ? 128 : 64;   // 128 bytes of K per LDS row for either element size
+  const int64_t cus = 256;
   a->group_m = 8;
   a->split_k = 1;
-  if (a->m <= 64) {
-    // skinny: B is streamed once, K is split until the grid covers the chip a few times over
-    a->block_m = 64; a->block_n = 128; a->block_k = bk; a->num_stages = 3; a->num_warps = 4;
+  a->block_k = bk;
+  bool dma_ok;
+  {
+    tnx_gemm_args t = *a;
+    t.a = t.b = nullptr;
+    if (t.stride_ak == 0 && t.stride_bn == 0) { t.stride_am = t.k; t.stride_ak = 1; t.stride_bk = t.n; t.stride_bn = 1; }
+    t.block_m = 128; t.block_n = 128; t.block_k = bk;
+    dma_ok = fast_layout(&t);
+  }
+  if (a->m <= 64 && dma_ok) {
+    // skinny: B is streamed once, K is split until the grid covers the chip about twice
+    a->block_m = 64; a->block_n = 128; a->num_stages = 3; a->num_warps = 4;
     int64_t tiles = (a->n + a->block_n - 1) / a->block_n;
     int64_t kt = (a->k + a->block_k - 1) / a->block_k;
     int s = 1;
-    while (tiles * s < 512 && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
+    while (tiles * s < 2 * cus && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
     a->split_k = s;
-  } else if (a->m >= 2048 && a->n >= 2048) {
-    // two waves per SIMD fill each other's issue gaps on the 256x256 tile
-    a->block_m = 256; a->block_n = 256; a->block_k = bk; a->num_stages = 2; a->num_warps = 8;
-  } else {
-    a->block_m = 128; a->block_n = 128; a->block_k = bk; a->num_stages = 3; a->num_warps = 4;
+    return TNX_OK;
+  }
+  // largest tile that still gives every CU a workgroup; two waves per SIMD on the big tiles
+  // fill each other's issue gaps
+  // operands the DMA loader cannot take (ragged K, odd strides or widths) go to one of the two
+  // tiles that are also built with the element-wise loader
+  if (!dma_ok) {
+    a->block_m = a->m <= 64 ? 64 : 128; a->block_n = 128; a->num_stages = 2; a->num_warps = 4;
+    return TNX_OK;
+  }
+  static const int cand[][4] = {{256, 256, 2, 8}, {256, 128, 3, 8}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
+  const int ncand = es == 1 ? 4 : 5;   // int8 rows of a 64-wide B tile are too short for the transposing read
+  for (int i = 0; i < ncand; ++i) {
+    a->block_m = cand[i][0]; a->block_n = cand[i][1]; a->num_stages = cand[i][2]; a->num_warps = cand[i][3];
+    int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
+    if (tiles >= cus * 3 / 4) break;
   }
   return TNX_OK;
 }

@@ -40,7 +40,7 @@ struct GemmParams {
   const uint8_t* a;
   const uint8_t* b;
   uint8_t* c;
-  uint8_t* ws;            // split-K partials [split][m][n], fp32 or int32
+  uint8_t* ws;            // split-K workspace: tile counters, then partials [split][m][n] (fp32 / int32)
   int64_t m, n, k;
   int64_t sam, sak;       // element strides of A
   int64_t sbk, sbn;       // element strides of B
@@ -139,6 +139,24 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
   uint64_t v = (uint64_t)(uintptr_t)p;
   uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Device-scope (all XCDs) 16-byte and 4-byte accesses for data that workgroups hand to each
+// other inside one kernel: the sc1 bit writes through / reads around the per-XCD L2, so no
+// whole-cache write-back or invalidate is needed around them.
+__device__ __forceinline__ void store16_agent(void* dst, i32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ i32x4 load16_agent(const void* src) {
+  i32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(src) : "memory");
+  return v;
+}
+__device__ __forceinline__ void store4_agent(int* dst, int v) {
+  __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int load4_agent(const int* src) {
+  return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
@@ -256,7 +274,7 @@ template <class C, int OES> struct EpiStage {
 // and stores 16 bytes per lane, so every row of C receives full contiguous
 // runs instead of 8-byte fragments.  GLU != 0: columns (2c, 2c+1) hold
 // (gate, linear); output column c.
-template <class T, class C, class O, int GLU, class ACC>
+template <class T, class C, class O, int GLU, bool AGENT = false, class ACC>
 __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t lds_strip, int lane,
                                                int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
                                                int64_t scn, bool vec_ok, int epi) {
@@ -314,18 +332,107 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t
       if (gm >= m) continue;
       raw* dst = cp + gm * scm + gc * scn;
       if (vec_ok && gc + VEC <= ncols) {
-        *(i32x4*)dst = v;
+        if constexpr (AGENT) store16_agent(dst, v);
+        else *(i32x4*)dst = v;
       } else {
         raw e[VEC];
         __builtin_memcpy(e, &v, 16);
 #pragma unroll
         for (int x = 0; x < VEC; ++x)
-          if (gc + x < ncols) dst[x * scn] = e[x];
+          if (gc + x < ncols) {
+            if constexpr (AGENT) store4_agent((int*)dst + x * scn, __builtin_bit_cast(int, e[x]));
+            else dst[x * scn] = e[x];
+          }
       }
     }
     // the next row-block overwrites the strip: wait for the reads above
     __builtin_amdgcn_s_waitcnt(0xC07F);
   }
+}
+
+// The first WS_COUNTER_BYTES of the split-K workspace hold one arrival counter per output
+// tile.  They must be zero when a launch starts; every launch leaves them zero.
+constexpr int WS_COUNTER_BYTES = 65536;
+constexpr int WS_MAX_TILES = WS_COUNTER_BYTES / 4;
+
+// Split-K tail.  Every wave has just stored its partial with device-scope stores.  One lane
+// bumps the tile's counter, and the workgroup that finds the counter at split_k-1 owns the
+// reduction: it reads the slices back with device-scope loads, adds them in slice order (so
+// the result does not depend on arrival order), applies the epilogue, writes C and re-arms
+// the counter.  Whole-L2 write-backs and invalidates (what a device-scope fence costs on a
+// part with eight L2s) are avoided on purpose: they cost more than the GEMM.
+template <class T, class C>
+__device__ __forceinline__ void splitk_finish(const GemmParams& p, const typename T::acc_s* part, int* counter, int* flag,
+                                              int64_t m0, int64_t n0) {
+  typedef typename T::acc_s acc_s;
+  typedef typename OutOf<T>::type O;
+  typedef Cvt<O, acc_s> CV;
+  typedef typename CV::raw raw;
+  // the partial was written with device-scope stores: once this wave's stores are acknowledged
+  // they are visible to every XCD, so the arrival count may follow
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (*flag != p.split_k - 1) return;
+  const bool vec_in = (p.n & 3) == 0;
+  const bool glu = p.epilogue != EPI_NONE;
+  raw* cp = (raw*)p.c;
+  for (int idx = threadIdx.x; idx < C::BM * (C::BN / 4); idx += C::THREADS) {
+    const int row = idx / (C::BN / 4), c4 = idx % (C::BN / 4);
+    const int64_t gm = m0 + row, gn = n0 + c4 * 4;
+    if (gm >= p.m || gn >= p.n) continue;
+    acc_s v[4] = {0, 0, 0, 0};
+    // slices are fetched eight at a time (all loads in flight together), then added in slice order
+    for (int z0 = 0; z0 < p.split_k; z0 += 8) {
+      acc_s q[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int z = z0 + u < p.split_k ? z0 + u : p.split_k - 1;
+        const acc_s* src = part + ((int64_t)z * p.m + gm) * p.n + gn;
+        if (vec_in) {
+          const uint64_t lo = __hip_atomic_load((const uint64_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint64_t hi = __hip_atomic_load((const uint64_t*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          q[u][0] = __builtin_bit_cast(acc_s, (uint32_t)lo); q[u][1] = __builtin_bit_cast(acc_s, (uint32_t)(lo >> 32));
+          q[u][2] = __builtin_bit_cast(acc_s, (uint32_t)hi); q[u][3] = __builtin_bit_cast(acc_s, (uint32_t)(hi >> 32));
+        } else {
+#pragma unroll
+          for (int x = 0; x < 4; ++x)
+            q[u][x] = gn + x < p.n ? __builtin_bit_cast(acc_s, load4_agent((const int*)src + x)) : (acc_s)0;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (z0 + u < p.split_k) { v[0] += q[u][0]; v[1] += q[u][1]; v[2] += q[u][2]; v[3] += q[u][3]; }
+    }
+    if (glu) {
+      const int64_t nh = p.n >> 1, gc = gn >> 1;
+      raw* dst = cp + gm * p.scm + gc * p.scn;
+      raw z0 = CV::run((acc_s)(glu_gate((float)v[0], p.epilogue) * (float)v[1]));
+      raw z1 = CV::run((acc_s)(glu_gate((float)v[2], p.epilogue) * (float)v[3]));
+      if (gc < nh) dst[0] = z0;
+      if (gc + 1 < nh) dst[p.scn] = z1;
+    } else {
+      raw* dst = cp + gm * p.scm + gn * p.scn;
+      if (p.c_vec_ok && gn + 3 < p.n) {
+        raw r[4] = {CV::run(v[0]), CV::run(v[1]), CV::run(v[2]), CV::run(v[3])};
+        if constexpr (sizeof(raw) == 2) {
+          i32x2 pk;
+          __builtin_memcpy(&pk, r, 8);
+          *(i32x2*)dst = pk;
+        } else {
+          i32x4 pk;
+          __builtin_memcpy(&pk, r, 16);
+          *(i32x4*)dst = pk;
+        }
+      } else {
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+          if (gn + x < p.n) dst[x * p.scn] = CV::run(v[x]);
+      }
+    }
+  }
+  if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <bool B> struct BoolTag { static constexpr bool value = B; };
@@ -626,9 +733,14 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int64_t gm0 = m0 + wy * C::WTM;
   const int64_t gn0 = n0 + wx * C::WTN;
   if (p.split_k > 1) {
-    acc_s* ws = (acc_s*)p.ws + (int64_t)split * p.m * p.n;
+    // fp32 / int32 partial of this K slice -> workspace [split][m][n]; the workgroup that
+    // arrives last at the tile's counter sums all slices in slice order and writes C
+    acc_s* part = (acc_s*)(p.ws + WS_COUNTER_BYTES);
     const uint32_t strip = lds0 + wave * EpiStage<C, 4>::WAVE_BYTES;
-    epilogue_store<T, C, acc_s, 0>(acc, (uint8_t*)ws, strip, lane, gm0, gn0, p.m, p.n, p.n, 1, (p.n & 3) == 0, 0);
+    epilogue_store<T, C, acc_s, 0, true>(acc, (uint8_t*)(part + (int64_t)split * p.m * p.n), strip, lane, gm0, gn0, p.m, p.n,
+                                   p.n, 1, (p.n & 3) == 0, 0);
+    splitk_finish<T, C>(p, part, (int*)p.ws + logical, (int*)smem, m0, n0);
+    return;
   } else {
     typedef typename OutOf<T>::type O;
     const uint32_t strip = lds0 + wave * EpiStage<C, sizeof(typename Cvt<O, acc_s>::raw)>::WAVE_BYTES;
@@ -636,33 +748,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       epilogue_store<T, C, O, 0>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
     else
       epilogue_store<T, C, O, 1>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
-  }
-}
-
-// ---------------------------------------------------------------------------
-// split-K second pass: sum the partials in a fixed order, then apply the
-// epilogue.  One thread per output element.
-// ---------------------------------------------------------------------------
-template <class ACC>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const ACC* __restrict__ ws, uint8_t* c, int64_t m, int64_t n,
-                                                            int64_t scm, int64_t scn, int split_k, int epilogue,
-                                                            int out_dtype) {
-  const int64_t ncols = epilogue == EPI_NONE ? n : n / 2;
-  const int64_t total = m * ncols;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    int64_t gm = idx / ncols, gc = idx % ncols;
-    if (epilogue == EPI_NONE) {
-      ACC s = 0;
-      for (int z = 0; z < split_k; ++z) s += ws[((int64_t)z * m + gm) * n + gc];
-      store_out<ACC>(c, gm * scm + gc * scn, s, out_dtype);
-    } else {
-      float g = 0.f, l = 0.f;
-      for (int z = 0; z < split_k; ++z) {
-        g += (float)ws[((int64_t)z * m + gm) * n + 2 * gc];
-        l += (float)ws[((int64_t)z * m + gm) * n + 2 * gc + 1];
-      }
-      store_out<float>(c, gm * scm + gc * scn, glu_gate(g, epilogue) * l, out_dtype);
-    }
   }
 }
 

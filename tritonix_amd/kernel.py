@@ -48,13 +48,16 @@ def out_dtype_for(dtype):
 
 
 def _workspace(device, stream_ptr: int, nbytes: int):
-    """Split-K scratch, one growing buffer per (device, stream); contents never need initialising."""
+    """Split-K scratch, one growing buffer per (device, stream).
+
+    Allocated zero-filled: the leading counter region must start at zero and every launch leaves it zero.
+    """
     import torch
 
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
 
@@ -145,17 +148,57 @@ class HipKernel:
 
         lib = _C.load()
         g = self.make_args(bound)
-        with torch.cuda.device(a.device):
-            stream = torch.cuda.current_stream(a.device).cuda_stream
-            g.stream = stream
-            if g.split_k > 1:
-                need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
-                if need:
-                    ws = _workspace(a.device, stream, need)
-                    g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
-            status = lib.tnx_gemm(ctypes.byref(g))
+        if a.device.index != torch.cuda.current_device():
+            with torch.cuda.device(a.device):
+                status = self._launch(lib, g, a.device)
+        else:
+            status = self._launch(lib, g, a.device)
         _C.raise_for_status(status, g)
         return None
+
+    @staticmethod
+    def _launch(lib, g, device) -> int:
+        import torch
+
+        stream = torch.cuda.current_stream(device).cuda_stream
+        g.stream = stream
+        if g.split_k > 1:
+            need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
+            if need:
+                ws = _workspace(device, stream, need)
+                g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
+        return lib.tnx_gemm(ctypes.byref(g))
+
+    def prepare(self, *args, **kwargs) -> Callable[[], None]:
+        """Bind a launch once and return a zero-argument callable that repeats it.
+
+        The tensors, tile config, stream and split-K workspace are captured at bind time; the returned
+        callable only performs the C-ABI call (for launch-bound shapes and for benchmarks).
+        """
+        import torch
+
+        bound = self._bind(args, kwargs)
+        lib = _C.load()
+        g = self.make_args(bound)
+        device = bound["a"].device
+        stream = torch.cuda.current_stream(device).cuda_stream
+        g.stream = stream
+        keep = [bound["a"], bound["b"], bound["c"]]
+        if g.split_k > 1:
+            need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
+            ws = _workspace(device, stream, need)
+            g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
+            keep.append(ws)
+        status = lib.tnx_gemm_supported(ctypes.byref(g))
+        _C.raise_for_status(status, g)
+        ref, fn = ctypes.byref(g), lib.tnx_gemm
+
+        def launch(_keep=keep, _g=g):
+            st = fn(ref)
+            if st:
+                _C.raise_for_status(st, _g)
+
+        return launch
 
     # host-only helpers -------------------------------------------------
     def lds_bytes(self, in_dtype_code: int, block_m: int, block_n: int, block_k: int, num_stages: int) -> int:

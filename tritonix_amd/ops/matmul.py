@@ -133,6 +133,8 @@ def default_config(a, b, split=False):
     g = _C.GemmArgs()
     g.m, g.k = a.shape
     g.n = b.shape[1]
+    g.stride_am, g.stride_ak = a.stride()
+    g.stride_bk, g.stride_bn = b.stride()
     g.in_dtype = _torch_dtype_code(a.dtype)
     _C.load().tnx_gemm_default_config(ctypes.byref(g))
     cfg = {"block_m": g.block_m, "block_n": g.block_n, "block_k": g.block_k, "group_m": g.group_m,
