@@ -23,8 +23,10 @@ import time
 PEAK = {"bf16": 2516.6, "f16": 2516.6, "i8": 5033.2}     # dense MFMA TFLOP/s (TOP/s), MI355X
 HBM_PEAK_GBS = 8000.0
 
-# measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the headline kernel; see profiles/
-TRAFFIC_BYTES_C2 = None
+# L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# (KiB per dispatch), each scaled by what the same counter reads for bench.py's 2^28-byte calibration pass:
+# (789484.6 * 2.0 + 131072.0 * 1.0) KiB.  See profiles/gemm_tile_bf16_256x256x64_c2_8192.md.
+TRAFFIC_BYTES_C2 = int((789484.6 * 2.0 + 131072.0 * 1.0) * 1024)
 
 
 def parse():
@@ -84,11 +86,11 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
 
-    # one plain device copy of known size (2^28 bytes read, 2^28 written): under `rocprofv3 --pmc
-    # FETCH_SIZE` / `WRITE_SIZE` it is the dispatch the GEMM's counter readings are scaled by
-    cal_src = torch.empty(1 << 28, dtype=torch.uint8, device=dev)
+    # one plain elementwise pass of known size (2^28 bytes read, 2^28 bytes written): under
+    # `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` it is the dispatch the GEMM's counter readings are scaled by
+    cal_src = torch.zeros(1 << 26, dtype=torch.int32, device=dev)
     cal_dst = torch.empty_like(cal_src)
-    cal_dst.copy_(cal_src)
+    torch.add(cal_src, 1, out=cal_dst)
     torch.cuda.synchronize()
     del cal_src, cal_dst
 
