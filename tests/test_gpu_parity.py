@@ -224,3 +224,25 @@ def test_error_mapping_on_launch(device):
         gemm(a.float(), a.float(), GENERIC)
     with pytest.raises(ValueError):
         gemm(a.cpu(), a.cpu(), GENERIC)
+
+
+# ---- wavefront-level split-K kernel (m <= 16, eight K slices meet in LDS) ---------------
+@pytest.mark.parametrize("m,n,k,stages,dtype", [(16, 4096, 14336, 6, torch.bfloat16), (16, 512, 2048, 3, torch.bfloat16),
+                                                (5, 96, 512, 4, torch.bfloat16), (1, 32, 256, 5, torch.float16)])
+def test_skinny_wave_split_kernel(device, m, n, k, stages, dtype):
+    if (m, n, k) == (16, 4096, 14336):
+        a, b = oracle.make_inputs("C3")
+    else:
+        g = torch.Generator("cpu").manual_seed(m * 7 + n)
+        a = torch.randn(m, k, generator=g).to(dtype)
+        b = (0.05 * torch.randn(k, n, generator=g)).to(dtype)
+    config = dict(block_m=16, block_n=32, block_k=32, group_m=8, split_k=8, num_stages=stages, num_warps=8)
+    out = gemm(a.to(device), b.to(device), config, kernel=gemm_splitk_kernel)
+    check_fp(out, oracle.reference_matmul(a, b))
+    assert torch.equal(gemm(a.to(device), b.to(device), config, kernel=gemm_splitk_kernel), out)
+    with pytest.raises(ValueError):      # this kernel is the eight-way split: nothing else is accepted
+        gemm(a.to(device), b.to(device), dict(config, split_k=4), kernel=gemm_splitk_kernel)
+    if m < 17:
+        with pytest.raises(ValueError):  # and it only takes up to sixteen rows
+            big = torch.zeros(17, k, dtype=dtype, device=device)
+            gemm(big, b.to(device), config, kernel=gemm_splitk_kernel)

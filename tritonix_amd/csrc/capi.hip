@@ -31,8 +31,13 @@ static const KernelEntry* find_entry(const tnx_gemm_args* a) {
 static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 // LDS bytes of a tile config, whether or not a kernel is built for it
+static bool is_skinny_cfg(const tnx_gemm_args* a) {
+  return a->block_m == SKINNY_BM && a->block_n == SKINNY_BN && a->block_k == SKINNY_BK && a->num_warps == SKINNY_NW;
+}
+
 static int64_t lds_bytes_of(const tnx_gemm_args* a) {
   if (a->block_m <= 0 || a->block_n <= 0 || a->block_k <= 0 || a->num_stages <= 0) return -1;
+  if (is_skinny_cfg(a)) return (int64_t)a->num_stages * SKINNY_NW * SKINNY_STEP_BYTES;
   int es = elem_size(a->in_dtype);
   return (int64_t)a->num_stages * ((int64_t)a->block_m * a->block_k + (int64_t)a->block_k * a->block_n) * es;
 }
@@ -75,6 +80,7 @@ extern "C" int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* a) {
 
 extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
   if (!a || a->split_k <= 1 || a->m <= 0 || a->n <= 0) return 0;
+  if (is_skinny_cfg(a)) return 0;   // the eight K slices meet in LDS
   return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)a->m * (size_t)a->n * 4;
 }
 
@@ -83,6 +89,22 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   if (st != TNX_OK) return st;
   int64_t lds = lds_bytes_of(a);
   if (lds > TNX_LDS_LIMIT_BYTES) return TNX_E_LDS;
+  if (is_skinny_cfg(a)) {
+    // m <= 16 rows, K cut eight ways inside the workgroup, DMA loader only
+    if (a->split_k != SKINNY_SPLIT || a->epilogue != TNX_EPI_NONE || a->in_dtype == TNX_I8) return TNX_E_UNSUPPORTED;
+    if (!skinny_lookup(a->in_dtype, a->num_stages)) return TNX_E_UNSUPPORTED;
+    if (a->m > SKINNY_BM || a->m < 1 || a->n % SKINNY_BN != 0 || a->k % (SKINNY_SPLIT * SKINNY_BK) != 0 || a->k == 0)
+      return TNX_E_UNSUPPORTED;
+    if (a->stride_ak != 1 || a->stride_bn != 1 || (a->stride_am * 2) % 16 != 0 || (a->stride_bk * 2) % 16 != 0 ||
+        a->stride_am < 0 || a->stride_bk < 0)
+      return TNX_E_UNSUPPORTED;
+    if (inspect_ptrs && ((((uintptr_t)a->a) & 15) || (((uintptr_t)a->b) & 15))) return TNX_E_UNSUPPORTED;
+    if ((int64_t)SKINNY_BK * a->stride_bk * 2 >= (1ll << 32) || (int64_t)SKINNY_BM * a->stride_am * 2 >= (1ll << 32))
+      return TNX_E_UNSUPPORTED;
+    if (out) *out = nullptr;
+    if (fast) *fast = true;
+    return TNX_OK;
+  }
   const KernelEntry* e = find_entry(a);
   if (!e) return TNX_E_UNSUPPORTED;
   tnx_gemm_args tmp = *a;
@@ -109,7 +131,8 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
     if (!a->c || (a->k > 0 && (!a->a || !a->b))) return TNX_E_INVALID;
   }
   if (a->m == 0 || a->n == 0) return TNX_OK;
-  if (a->split_k > 1 && (!a->workspace || a->workspace_bytes < tnx_gemm_workspace_bytes(a) || ((uintptr_t)a->workspace & 255)))
+  if (tnx_gemm_workspace_bytes(a) > 0 &&
+      (!a->workspace || a->workspace_bytes < tnx_gemm_workspace_bytes(a) || ((uintptr_t)a->workspace & 255)))
     return TNX_E_WORKSPACE;
 
   const int es_out = elem_size(a->out_dtype);
@@ -134,8 +157,13 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.c_vec_ok = a->stride_cn == 1 && ((a->stride_cm * es_out) % 16) == 0 && (((uintptr_t)a->c) % 16) == 0;
 
   hipStream_t stream = (hipStream_t)a->stream;
-  unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * a->split_k);
-  hipError_t err = (fast ? e->fast : e->generic)(p, grid, stream);
+  hipError_t err;
+  if (is_skinny_cfg(a)) {
+    err = skinny_lookup(a->in_dtype, a->num_stages)(p, (unsigned)(a->n / SKINNY_BN), stream);
+  } else {
+    unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * a->split_k);
+    err = (fast ? e->fast : e->generic)(p, grid, stream);
+  }
   if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
 
   return TNX_OK;
@@ -158,17 +186,16 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     dma_ok = fast_layout(&t);
   }
   if (a->m <= 64 && dma_ok) {
-    // skinny: B is streamed once, K is split until the grid covers the chip about twice
-    a->block_m = 64; a->block_n = 128; a->num_stages = 3; a->num_warps = 4;
+    // skinny: B is streamed once; K is split until every CU owns one workgroup (measured on the
+    // M=16, N=4096, K=14336 shape: 8 waves, 3 stages, 256 workgroups stream at the HBM read limit)
+    a->block_m = 64; a->block_n = 128; a->num_stages = 3; a->num_warps = 8;
     int64_t tiles = (a->n + a->block_n - 1) / a->block_n;
     int64_t kt = (a->k + a->block_k - 1) / a->block_k;
     int s = 1;
-    while (tiles * s < 2 * cus && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
+    while (tiles * s < cus && s * 2 <= 16 && kt / (s * 2) >= 4) s *= 2;
     a->split_k = s;
     return TNX_OK;
   }
-  // largest tile that still gives every CU a workgroup; two waves per SIMD on the big tiles
-  // fill each other's issue gaps
   // operands the DMA loader cannot take (ragged K, odd strides or widths) go to one of the two
   // tiles that are also built with the element-wise loader
   if (!dma_ok) {

@@ -28,6 +28,12 @@ hipError_t launch_tile(const GemmParams& p, unsigned grid, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// skinny kernel (gemm_skinny.h): tile 16 x 32 x 32, eight waves, split_k == 8 inside the workgroup,
+// num_stages = ring depth per wave.  Null when that depth / dtype is not built.
+launch_fn skinny_lookup(int dtype, int ring);
+constexpr int SKINNY_BM = 16, SKINNY_BN = 32, SKINNY_BK = 32, SKINNY_NW = 8, SKINNY_SPLIT = 8;
+constexpr int SKINNY_STEP_BYTES = 3072;
+
 #define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
   {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
    &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \

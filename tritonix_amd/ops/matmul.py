@@ -55,12 +55,12 @@ matmul_kernel = tunable(
 gemm_splitk_kernel = tunable(
     keys=["m", "n", "k"],
     space={
-        "block_m": PowerOfTwo(64, 128),
-        "block_n": PowerOfTwo(64, 256),
+        "block_m": PowerOfTwo(16, 128),
+        "block_n": PowerOfTwo(32, 256),
         "block_k": PowerOfTwo(32, 128),
         "group_m": Choice([4, 8]),
         "split_k": PowerOfTwo(2, 16),
-        "num_stages": Range(2, 4),
+        "num_stages": Range(2, 6),
         "num_warps": Choice([4, 8]),
     },
     memory_params={"block_m", "block_n", "block_k", "num_stages"},
