@@ -695,7 +695,25 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   }
 
   int t = 0;
-  // (1) periods that issue the refill of slab t+STAGES into the slot of slab t
+  // (1) periods that issue the refill of slab t+STAGES into the slot of slab t.  The bulk runs
+  // STAGES periods per trip so every ring slot is a compile-time constant there (LDS addresses
+  // become instruction immediates, DMA targets become scalar constants); what is left over runs
+  // with run-time slots.
+  if constexpr (FAST) {
+    for (; t + 2 * STAGES - 1 < KT; t += STAGES) {
+#pragma unroll
+      for (int j = 0; j < STAGES; ++j) {
+        __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t dst = lds0 + (uint32_t)j * C::STAGE_BYTES;
+        const uint32_t sa1 = lds0 + (uint32_t)((j + 1) % STAGES) * C::STAGE_BYTES, sb1 = sa1 + C::A_BYTES;
+        last_step(sa1, sb1, Yes{}, dst);
+        inner_steps(sa1, sb1, Yes{}, dst);
+        dma_advance();
+      }
+    }
+  }
   for (; t + STAGES < KT; ++t) {
     __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
     __builtin_amdgcn_s_barrier();
