@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--tune", action="store_true", help="run the grid tuner for each workload instead of the built-in tiles")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--tile", default=None, help="headline tile override: block_m,block_n,block_k,num_warps,num_stages,group_m")
     return ap.parse_args()
 
 
@@ -101,6 +102,9 @@ def main():
     n = b.shape[1]
     flops = 2.0 * m * n * k
     cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+    if args.tile:
+        bm, bn, bk, nw, st, gm = (int(v) for v in args.tile.split(","))
+        cfg = {"block_m": bm, "block_n": bn, "block_k": bk, "group_m": gm, "num_stages": st, "num_warps": nw}
     c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
     grid = (-(-m // cfg["block_m"]), -(-n // cfg["block_n"]))
 

@@ -202,7 +202,7 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     a->block_m = a->m <= 64 ? 64 : 128; a->block_n = 128; a->num_stages = 2; a->num_warps = 4;
     return TNX_OK;
   }
-  static const int cand[][4] = {{256, 256, 2, 8}, {256, 128, 3, 8}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
+  static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
   const int ncand = es == 1 ? 4 : 5;   // int8 rows of a 64-wide B tile are too short for the transposing read
   for (int i = 0; i < ncand; ++i) {
     a->block_m = cand[i][0]; a->block_n = cand[i][1]; a->num_stages = cand[i][2]; a->num_warps = cand[i][3];

@@ -245,7 +245,10 @@ struct TileCfg {
 // ---------------------------------------------------------------------------
 // output conversion and the store of a wave's accumulators
 // ---------------------------------------------------------------------------
-struct OutBF16 { typedef uint16_t raw; static __device__ __forceinline__ raw cvt(float v) { return f32_to_bf16(v); } };
+struct OutBF16 {
+  typedef uint16_t raw;
+  static __device__ __forceinline__ raw cvt(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }  // RNE
+};
 struct OutF16 {
   typedef uint16_t raw;
   static __device__ __forceinline__ raw cvt(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
@@ -255,93 +258,107 @@ template <> struct OutOf<TagBF16> { typedef OutBF16 type; };
 template <> struct OutOf<TagF16> { typedef OutF16 type; };
 template <> struct OutOf<TagI8> { typedef int type; };
 
-template <class O, class S> struct Cvt { typedef typename O::raw raw; static __device__ __forceinline__ raw run(S v) { return O::cvt((float)v); } };
-template <> struct Cvt<float, float> { typedef float raw; static __device__ __forceinline__ float run(float v) { return v; } };
-template <> struct Cvt<int, int> { typedef int raw; static __device__ __forceinline__ int run(int v) { return v; } };
+template <class O, class S> struct Cvt1 { typedef typename O::raw raw; static __device__ __forceinline__ raw run(S v) { return O::cvt((float)v); } };
+template <> struct Cvt1<int, int> { typedef int raw; static __device__ __forceinline__ int run(int v) { return v; } };
 
-// Bytes of LDS one wave needs to transpose one row-block (MI rows) of its
-// output through LDS; rows are padded by 16 bytes to spread the banks.
-template <class C, int OES> struct EpiStage {
-  static constexpr int PITCH = C::WTN * OES + 16;
+// LDS one wave needs to pass one row-block (MI rows) of its accumulators through LDS: raw
+// 32-bit values, rows padded by 16 bytes to spread the banks.
+template <class C> struct EpiStage {
+  static constexpr int PITCH = C::WTN * 4 + 16;
   static constexpr int WAVE_BYTES = C::MI * PITCH;
   static constexpr int BYTES = C::NW * WAVE_BYTES;
 };
 
-// The MFMA result is C^T: lane l owns output row m = l % MI and, per group of
-// four accumulator registers, four consecutive columns n.  Each wave writes
-// one row-block at a time into its private LDS strip ([MI rows][wave-tile
-// columns], output dtype, gating already applied), reads it back row-major
-// and stores 16 bytes per lane, so every row of C receives full contiguous
-// runs instead of 8-byte fragments.  GLU != 0: columns (2c, 2c+1) hold
-// (gate, linear); output column c.
-template <class T, class C, class O, int GLU, bool AGENT = false, class ACC>
+// 16 bytes of output from NF accumulator values that sit row-major in LDS.
+// GLU: values come in (gate, linear) pairs, one output per pair.
+template <class O, class S, bool GLU> struct Pack16;
+template <class O, bool GLU> struct Pack16<O, float, GLU> {   // 16-bit float outputs: 8 per lane
+  typedef typename O::raw raw;
+  static constexpr int OUTV = 8, NF = GLU ? 16 : 8;
+  static __device__ __forceinline__ void run(const float* f, int epi, raw* out) {
+#pragma unroll
+    for (int x = 0; x < OUTV; ++x) out[x] = O::cvt(GLU ? glu_gate(f[2 * x], epi) * f[2 * x + 1] : f[x]);
+  }
+};
+template <bool GLU> struct Pack16<float, float, GLU> {        // fp32 outputs (split-K partials): 4 per lane
+  typedef float raw;
+  static constexpr int OUTV = 4, NF = 4;
+  static __device__ __forceinline__ void run(const float* f, int, raw* out) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = f[x];
+  }
+};
+template <bool GLU> struct Pack16<int, int, GLU> {            // int32 outputs: 4 per lane
+  typedef int raw;
+  static constexpr int OUTV = 4, NF = 4;
+  static __device__ __forceinline__ void run(const int* f, int, raw* out) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = f[x];
+  }
+};
+
+// The MFMA result is C^T: lane l owns output row m = l % MI and, per group of four accumulator
+// registers, four consecutive columns n.  Each wave passes one row-block at a time through its
+// private LDS strip: raw accumulators in (one ds_write_b128 per group, nothing else in the
+// unrolled part), then a plain loop reads the strip row-major, converts / gates, and stores 16
+// bytes per lane, so every row of C receives full contiguous runs.  Keeping the conversion out
+// of the unrolled part keeps the three epilogue variants of a 256x256 tile inside the
+// instruction cache.
+template <class T, class C, class O, bool GLU, bool AGENT, class ACC>
 __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t lds_strip, int lane,
                                                int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
                                                int64_t scn, bool vec_ok, int epi) {
   typedef typename T::acc_s acc_s;
-  typedef Cvt<O, acc_s> CV;
-  typedef typename CV::raw raw;
+  typedef Pack16<O, acc_s, GLU> PK;
+  typedef typename PK::raw raw;
+  typedef acc_s acc4 __attribute__((ext_vector_type(4)));
   constexpr int MI = C::MI;
-  constexpr int OES = sizeof(raw);
   constexpr int NGRP = C::ACC_N / 4;                    // groups of four consecutive columns per accumulator tile
+  constexpr int PITCH = EpiStage<C>::PITCH;
   constexpr int WCOLS = GLU ? C::WTN / 2 : C::WTN;      // output columns of the wave tile
-  constexpr int PITCH = C::WTN * OES + 16;              // strip pitch (sized for the non-GLU case)
-  constexpr int VEC = 16 / OES;                         // elements per 16-byte store
-  constexpr int CPRW = WCOLS / VEC;                     // 16-byte chunks per strip row
+  constexpr int CPRW = WCOLS / PK::OUTV;                // 16-byte output chunks per strip row
   constexpr int ITERS = (MI * CPRW + 63) / 64;
-  static_assert(WCOLS % VEC == 0, "wave tile too narrow for 16-byte stores");
+  static_assert(WCOLS % PK::OUTV == 0, "wave tile too narrow for 16-byte stores");
   raw* cp = (raw*)cbase;
-  const int wrow = lane % MI, wcol = (lane / MI) * 4;
+  const uint32_t wbase = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
-    // ---- registers -> strip
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
+    for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-      for (int g = 0; g < NGRP; ++g) {
-        const int col = j * MI + g * 8 + wcol;          // column inside the wave tile (interleaved width)
-        acc_s v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
-        if constexpr (GLU) {
-          raw z0 = CV::run((acc_s)(glu_gate((float)v0, epi) * (float)v1));
-          raw z1 = CV::run((acc_s)(glu_gate((float)v2, epi) * (float)v3));
-          const uint32_t dst = lds_strip + wrow * PITCH + (col >> 1) * OES;
-          if constexpr (OES == 2) *TNX_LDS(uint32_t, dst) = (uint32_t)z0 | ((uint32_t)z1 << 16);
-          else *TNX_LDS(i32x2, dst) = i32x2{__builtin_bit_cast(int, z0), __builtin_bit_cast(int, z1)};
-        } else {
-          raw r0 = CV::run(v0), r1 = CV::run(v1), r2 = CV::run(v2), r3 = CV::run(v3);
-          const uint32_t dst = lds_strip + wrow * PITCH + col * OES;
-          if constexpr (OES == 2)
-            *TNX_LDS(i32x2, dst) = i32x2{(int)((uint32_t)r0 | ((uint32_t)r1 << 16)), (int)((uint32_t)r2 | ((uint32_t)r3 << 16))};
-          else
-            *TNX_LDS(i32x4, dst) = i32x4{__builtin_bit_cast(int, r0), __builtin_bit_cast(int, r1),
-                                         __builtin_bit_cast(int, r2), __builtin_bit_cast(int, r3)};
-        }
-      }
-    }
+      for (int g = 0; g < NGRP; ++g)
+        // (typed vector store: __builtin_bit_cast on an ext-vector element reads element 0)
+        *TNX_LDS(acc4, wbase + (j * MI + g * 8) * 4) =
+            acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
     // the strip is private to this wave: its own LDS writes are ordered before its reads
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    // ---- strip -> global, row-major 16-byte chunks
-#pragma unroll
+#pragma unroll 1
     for (int it = 0; it < ITERS; ++it) {
       const int q = it * 64 + lane;
       const int row = q / CPRW, cc = q % CPRW;
-      if (MI * CPRW % 64 != 0 && row >= MI) continue;
       const int64_t gm = gm0 + i * MI + row;
-      const int64_t gc = gc0 + cc * VEC;
-      i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + cc * 16);
-      if (gm >= m) continue;
+      const int64_t gc = gc0 + cc * PK::OUTV;
+      if ((MI * CPRW % 64 != 0 && row >= MI) || gm >= m) continue;
+      acc_s f[PK::NF];
+#pragma unroll
+      for (int x = 0; x < PK::NF / 4; ++x) {
+        const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * PK::NF + 4 * x) * 4);
+        __builtin_memcpy(&f[4 * x], &v, 16);
+      }
+      raw out[PK::OUTV];
+      PK::run(f, epi, out);
       raw* dst = cp + gm * scm + gc * scn;
-      if (vec_ok && gc + VEC <= ncols) {
+      if (vec_ok && gc + PK::OUTV <= ncols) {
+        i32x4 v;
+        __builtin_memcpy(&v, out, 16);
         if constexpr (AGENT) store16_agent(dst, v);
         else *(i32x4*)dst = v;
       } else {
-        raw e[VEC];
-        __builtin_memcpy(e, &v, 16);
-#pragma unroll
-        for (int x = 0; x < VEC; ++x)
+#pragma unroll 1
+        for (int x = 0; x < PK::OUTV; ++x)
           if (gc + x < ncols) {
-            if constexpr (AGENT) store4_agent((int*)dst + x * scn, __builtin_bit_cast(int, e[x]));
-            else dst[x * scn] = e[x];
+            if constexpr (AGENT) store4_agent((int*)dst + x * scn, __builtin_bit_cast(int, out[x]));
+            else dst[x * scn] = out[x];
           }
       }
     }
@@ -366,7 +383,7 @@ __device__ __forceinline__ void splitk_finish(const GemmParams& p, const typenam
                                               int64_t m0, int64_t n0) {
   typedef typename T::acc_s acc_s;
   typedef typename OutOf<T>::type O;
-  typedef Cvt<O, acc_s> CV;
+  typedef Cvt1<O, acc_s> CV;
   typedef typename CV::raw raw;
   // the partial was written with device-scope stores: once this wave's stores are acknowledged
   // they are visible to every XCD, so the arrival count may follow
@@ -448,7 +465,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
 
-  constexpr int SMEM_BYTES = C::LDS_BYTES > EpiStage<C, 4>::BYTES ? C::LDS_BYTES : EpiStage<C, 4>::BYTES;
+  constexpr int SMEM_BYTES = C::LDS_BYTES > EpiStage<C>::BYTES ? C::LDS_BYTES : EpiStage<C>::BYTES;
   __shared__ __attribute__((aligned(1024))) uint8_t smem[SMEM_BYTES];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
 
@@ -618,7 +635,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // to issue / ring draining / final step) so the accumulators flow through
   // straight-line code.
   constexpr int PERIOD = C::KSTEPS * NMMA;                       // MFMA slots per period
-  constexpr int SPAN = (STAGES == 2 || !FAST) ? NMMA : PERIOD;   // slots the refill is spread over
+  // slots the refill is spread over.  Two-slab rings: the refill is due at the next barrier, so it
+  // is front-loaded; with one wave per SIMD a single k step of DMA issue backs up the texture
+  // address queue (measured: 2630 -> 2210 cycles per slab when spread over two), with two waves
+  // per SIMD the other wave already covers the stall.
+  constexpr int SPAN2 = (NW == 4 && 2 * NMMA <= PERIOD) ? 2 * NMMA : NMMA;
+  constexpr int SPAN = (STAGES == 2 || !FAST) ? SPAN2 : PERIOD;
   constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
   constexpr int NEXT0 = C::KSTEPS & 1;                           // set that receives step 0 of the next slab
 
@@ -750,22 +772,22 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   __syncthreads();
   const int64_t gm0 = m0 + wy * C::WTM;
   const int64_t gn0 = n0 + wx * C::WTN;
+  const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
   if (p.split_k > 1) {
     // fp32 / int32 partial of this K slice -> workspace [split][m][n]; the workgroup that
     // arrives last at the tile's counter sums all slices in slice order and writes C
     acc_s* part = (acc_s*)(p.ws + WS_COUNTER_BYTES);
-    const uint32_t strip = lds0 + wave * EpiStage<C, 4>::WAVE_BYTES;
-    epilogue_store<T, C, acc_s, 0, true>(acc, (uint8_t*)(part + (int64_t)split * p.m * p.n), strip, lane, gm0, gn0, p.m, p.n,
-                                   p.n, 1, (p.n & 3) == 0, 0);
+    epilogue_store<T, C, acc_s, false, true>(acc, (uint8_t*)(part + (int64_t)split * p.m * p.n), strip, lane, gm0, gn0, p.m,
+                                             p.n, p.n, 1, (p.n & 3) == 0, 0);
     splitk_finish<T, C>(p, part, (int*)p.ws + logical, (int*)smem, m0, n0);
     return;
   } else {
     typedef typename OutOf<T>::type O;
-    const uint32_t strip = lds0 + wave * EpiStage<C, sizeof(typename Cvt<O, acc_s>::raw)>::WAVE_BYTES;
     if (p.epilogue == EPI_NONE)
-      epilogue_store<T, C, O, 0>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+      epilogue_store<T, C, O, false, false>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
     else
-      epilogue_store<T, C, O, 1>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
+      epilogue_store<T, C, O, true, false>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok,
+                                           p.epilogue);
   }
 }
 
