@@ -167,3 +167,30 @@ def test_default_configs_are_valid_and_correct(device, shape):
             assert torch.equal(out.cpu(), ref)
         else:
             assert oracle.within_tolerance(out, ref)[0]
+
+
+def test_swiglu_ffn(device):
+    from tritonix_amd.ops.swiglu import swiglu_ffn
+
+    x, w12 = oracle.make_inputs("C4", scale_down=16)          # x[256,256], w12[256,1792]
+    g = torch.Generator("cpu").manual_seed(44)
+    w3 = (0.05 * torch.randn(w12.shape[1] // 2, 320, generator=g)).bfloat16()
+    out = swiglu_ffn(x.to(device), w12.to(device), w3.to(device))
+    hidden = oracle.reference_glu(x, w12, "silu").bfloat16().float()   # the intermediate is stored in bf16
+    ok, _, rel = oracle.within_tolerance(out, hidden @ w3.float())
+    assert ok and rel <= 1e-2 and out.shape == (256, 320)
+    with pytest.raises(ValueError):
+        swiglu_ffn(x.to(device), w12.to(device), w3[:-1].to(device))
+
+
+def test_tuned_config_is_reused_from_disk(device, tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITONIX_CACHE_DIR", str(tmp_path))
+    a = torch.randn(384, 256, device=device, dtype=torch.float16)
+    b = torch.randn(256, 512, device=device, dtype=torch.float16)
+    mm._matmul_cfg.clear()
+    out1 = tritonix_amd.triton_matmul(a, b)
+    picked = mm._matmul_cfg[(384, 512, 256, torch.float16)]
+    assert mm.load_tuned("matmul", (384, 512, 256, torch.float16)) == picked
+    mm._matmul_cfg.clear()
+    monkeypatch.setattr(mm.matmul_kernel, "tune", lambda *a, **k: pytest.fail("tuned again despite the disk record"))
+    assert torch.equal(tritonix_amd.triton_matmul(a, b), out1)

@@ -32,7 +32,7 @@ from tritonix_amd.dispatcher import dynamic_dispatch
 from tritonix_amd.kernel import HipKernel, cdiv, out_dtype_for
 
 __all__ = ["matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel", "gemm_splitk_kernel",
-           "swizzle2d", "grouped_launch", "TUNE_OPTIONS"]
+           "swizzle2d", "grouped_launch", "TUNE_OPTIONS", "load_tuned", "save_tuned"]
 
 # keyword arguments handed to ``.tune`` on a config-memo miss (tests shrink the time budgets)
 TUNE_OPTIONS = {"warmup": 25, "rep": 100}
@@ -123,6 +123,71 @@ _matmul_cfg = {}
 _splitk_cfg = {}
 
 
+# ---------------------------------------------------------------------------
+# tuned tile configs on disk.  The reference only persists the dispatcher's backend winner
+# (tritonix/dispatcher.py:100-128) and re-tunes every process; here the tile config a grid
+# search picked is written next to it, one small JSON file per (op, shape, dtype).
+# ---------------------------------------------------------------------------
+def _tuned_path(op: str, key: tuple) -> str:
+    import hashlib
+
+    from tritonix_amd.dispatcher import cache_dir
+
+    digest = hashlib.sha256(f"{op}-{key}".encode()).hexdigest()
+    return os.path.join(cache_dir(), "tuned", digest + ".json")
+
+
+def load_tuned(op: str, key: tuple):
+    """Tile config stored for (op, key), or None.  ``TRITONIX_TUNE_CACHE=0`` switches the store off."""
+    import json
+
+    if os.environ.get("TRITONIX_TUNE_CACHE", "1") in ("0", "false", "False"):
+        return None
+    try:
+        with open(_tuned_path(op, key)) as f:
+            rec = json.load(f)
+        if rec.get("op") == op and rec.get("key") == [str(k) for k in key] and isinstance(rec.get("config"), dict):
+            return {k: int(v) for k, v in rec["config"].items()}
+    except (OSError, ValueError, TypeError):
+        pass
+    return None
+
+
+def save_tuned(op: str, key: tuple, cfg: dict) -> None:
+    import json
+    import tempfile
+
+    if os.environ.get("TRITONIX_TUNE_CACHE", "1") in ("0", "false", "False"):
+        return
+    try:
+        path = _tuned_path(op, key)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        fd, tmp = tempfile.mkstemp(dir=os.path.dirname(path), suffix=".tmp")
+        with os.fdopen(fd, "w") as f:
+            json.dump({"op": op, "key": [str(k) for k in key], "config": cfg}, f)
+        os.replace(tmp, path)
+    except OSError:
+        pass
+
+
+def _tuned_or_tune(op: str, key: tuple, kernel, launcher, fallback):
+    """Config for ``key``: disk record, else a grid search (stored afterwards), else the built-in choice."""
+    if not _autotune_enabled():
+        return fallback()
+    cfg = load_tuned(op, key)
+    if cfg is not None:
+        try:                      # a record written by another build may name a tile that no longer exists
+            launcher(cfg)
+            return cfg
+        except (ValueError, RuntimeError):
+            pass
+    cfg = kernel.tune(launcher, **TUNE_OPTIONS)
+    if cfg is None:
+        raise RuntimeError(f"no HIP tile kernel accepts {op} {key}")
+    save_tuned(op, key, cfg)
+    return cfg
+
+
 def default_config(a, b, split=False):
     """The engine's built-in tile choice for this problem (used when tuning is switched off)."""
     import ctypes
@@ -159,13 +224,8 @@ def triton_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     _, n = b.shape
     key = (m, n, k, a.dtype)
     if key not in _matmul_cfg:
-        if _autotune_enabled():
-            cfg = matmul_kernel.tune(lambda cfg: _launch_matmul(a, b, cfg), **TUNE_OPTIONS)
-            if cfg is None:
-                raise RuntimeError(f"no HIP tile kernel accepts {tuple(a.shape)} @ {tuple(b.shape)} {a.dtype}")
-            _matmul_cfg[key] = cfg
-        else:
-            _matmul_cfg[key] = default_config(a, b)
+        _matmul_cfg[key] = _tuned_or_tune("matmul", key, matmul_kernel, lambda cfg: _launch_matmul(a, b, cfg),
+                                          lambda: default_config(a, b))
     return _launch_matmul(a, b, _matmul_cfg[key])
 
 
@@ -183,13 +243,9 @@ def matmul_splitk(a: torch.Tensor, b: torch.Tensor, split_k: int = 4) -> torch.T
     _, n = b.shape
     key = (m, n, k, split_k, a.dtype)
     if key not in _splitk_cfg:
-        if _autotune_enabled():
-            cfg = gemm_splitk_kernel.tune(lambda cfg: _launch_splitk(a, b, cfg), **TUNE_OPTIONS)
-            if cfg is None:
-                raise RuntimeError(f"no HIP split-K kernel accepts {tuple(a.shape)} @ {tuple(b.shape)} {a.dtype}")
-            _splitk_cfg[key] = cfg
-        else:
-            _splitk_cfg[key] = default_config(a, b, split=True)
+        _splitk_cfg[key] = _tuned_or_tune("matmul_splitk", key, gemm_splitk_kernel,
+                                          lambda cfg: _launch_splitk(a, b, cfg),
+                                          lambda: default_config(a, b, split=True))
     return _launch_splitk(a, b, _splitk_cfg[key])
 
 

@@ -25,7 +25,7 @@ import importlib
 
 _mm = importlib.import_module("tritonix_amd.ops.matmul")  # the module: the package attribute `matmul` is the dispatcher
 
-__all__ = ["glu_kernel", "glu", "swiglu", "fused_glu", "silu", "interleave_weights"]
+__all__ = ["glu_kernel", "glu", "swiglu", "swiglu_ffn", "fused_glu", "silu", "interleave_weights"]
 
 glu_kernel = tunable(
     keys=["m", "n", "k"],
@@ -78,19 +78,27 @@ def glu(x: torch.Tensor, w12: torch.Tensor, activation: str = "silu") -> torch.T
     n = w12.shape[1]
     key = (m, n, k, x.dtype)
     if key not in _glu_cfg:
-        if _mm._autotune_enabled():
-            cfg = glu_kernel.tune(lambda cfg: _launch_glu(x, w12, cfg, activation), **_mm.TUNE_OPTIONS)
-            if cfg is None:
-                raise RuntimeError(f"no HIP GLU kernel accepts {tuple(x.shape)} @ {tuple(w12.shape)} {x.dtype}")
-            _glu_cfg[key] = cfg
-        else:
-            _glu_cfg[key] = _mm.default_config(x, w12)
+        _glu_cfg[key] = _mm._tuned_or_tune("glu", key, glu_kernel, lambda cfg: _launch_glu(x, w12, cfg, activation),
+                                           lambda: _mm.default_config(x, w12))
     return _launch_glu(x, w12, _glu_cfg[key], activation)
 
 
 def swiglu(x: torch.Tensor, w12: torch.Tensor) -> torch.Tensor:
     """SwiGLU up-projection: ``silu(x @ W1) * (x @ W2)`` with ``w12`` the interleaved ``[W1 | W2]``."""
     return glu(x, w12, activation="silu")
+
+
+def swiglu_ffn(x: torch.Tensor, w12: torch.Tensor, w3: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """SwiGLU feed-forward block ``(act(x @ W1) * (x @ W2)) @ W3``.
+
+    What the reference's draft ``swiglu_kernel`` is meant to compute (tritonix/ops/swiglu.py:127-230;
+    playground/swiglu.py:99-103).  The draft fuses the down-projection into the same kernel with atomic
+    adds and was never launched; here the gated up-projection is the fused GLU kernel and the
+    down-projection is the tiled GEMM, two launches with the [m, n] intermediate in the input dtype.
+    """
+    if w3.dim() != 2 or w3.shape[0] != w12.shape[1] // 2:
+        raise ValueError(f"w3 must be [{w12.shape[1] // 2}, f], got {tuple(w3.shape)}")
+    return _mm.triton_matmul(glu(x, w12, activation=activation), w3)
 
 
 def fused_glu(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
