@@ -25,8 +25,8 @@ HBM_PEAK_GBS = 8000.0
 
 # L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # (KiB per dispatch), each scaled by what the same counter reads for bench.py's 2^28-byte calibration pass:
-# (789484.6 * 2.0 + 131072.0 * 1.0) KiB.  See profiles/gemm_tile_bf16_256x256x64_c2_8192.md.
-TRAFFIC_BYTES_C2 = int((789484.6 * 2.0 + 131072.0 * 1.0) * 1024)
+# (844109.5 * 2.0 + 131072.0 * 1.0) KiB.  See profiles/gemm_tile_bf16_256x256x64_w4_c2_8192.md.
+TRAFFIC_BYTES_C2 = int((844109.5 * 2.0 + 131072.0 * 1.0) * 1024)
 
 
 def parse():
