@@ -10,7 +10,9 @@ one JSON line: whole-job TFLOP/s over the K timed steps, the roofline record
 of the kernel (algorithmic flops / mean per-launch duration from HIP events
 on the launch stream), the CPU baseline (torch fp32 matmul on the host
 cores, bounded sample) and, under "per_config", the other four benchmark
-configurations measured the same way.
+configurations measured the same way.  "vendor_ms" entries time torch's own
+GPU matmul (rocBLAS / hipBLASLt) on the same operands in the same run, for
+comparison only: nothing in the measured path calls it.
 """
 from __future__ import annotations
 
@@ -22,6 +24,7 @@ import time
 
 PEAK = {"bf16": 2516.6, "f16": 2516.6, "i8": 5033.2}     # dense MFMA TFLOP/s (TOP/s), MI355X
 HBM_PEAK_GBS = 8000.0
+PRE_ROLL = 40                                            # untimed launches that bring the part out of idle clocks
 
 # L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # (KiB per dispatch), each scaled by what the same counter reads for bench.py's 2^28-byte calibration pass:
@@ -37,6 +40,7 @@ def parse():
     ap.add_argument("--tune", action="store_true", help="run the grid tuner for each workload instead of the built-in tiles")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the rocBLAS/hipBLASLt timing of the same operands")
     ap.add_argument("--tile", default=None, help="headline tile override: block_m,block_n,block_k,num_warps,num_stages,group_m")
     return ap.parse_args()
 
@@ -53,6 +57,28 @@ def event_times(fn, n):
         stops[i].record()
     torch.cuda.synchronize()
     return [s.elapsed_time(e) for s, e in zip(starts, stops)]
+
+
+def cpu_time(fn, budget_s=8.0, max_reps=3):
+    """Median wall time of fn() on the host: one warm-up, then up to max_reps timed runs inside the budget."""
+    fn()
+    ts, t_start = [], time.perf_counter()
+    while len(ts) < max_reps and (not ts or time.perf_counter() - t_start < budget_s):
+        t1 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t1)
+    return sorted(ts)[len(ts) // 2], len(ts)
+
+
+def vendor_ms(fn, reps=20):
+    """Mean per-launch ms of a torch GPU op (the vendor BLAS), same event protocol as the kernels under test."""
+    import torch
+
+    for _ in range(PRE_ROLL):
+        fn(0)
+    torch.cuda.synchronize()
+    durs = event_times(fn, reps)
+    return round(sum(durs) / len(durs), 4)
 
 
 def pick_config(kernel, launcher, a, b, tune, split=False):
@@ -115,6 +141,10 @@ def main():
     def step(_i=0):
         launch()
 
+    # the clocks settle over the first few dozen launches after idle: run those before the W warm-up steps
+    for _ in range(PRE_ROLL):
+        step()
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -132,6 +162,14 @@ def main():
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK["bf16"], "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK["bf16"], 4), "traffic": TRAFFIC_BYTES_C2,
                 "kernel_ms": round(kern_ms, 4), "kernel_ms_min": round(min(durs), 4)}
+
+    vendor = None
+    if not args.no_vendor:
+        cv = torch.empty_like(c)
+        t = vendor_ms(lambda i: torch.matmul(a, b, out=cv))
+        vendor = {"what": "torch.matmul (rocBLAS/hipBLASLt) on the same operands, same run", "kernel_ms": t,
+                  "tflops": round(flops / t / 1e9, 1)}
+        del cv
 
     # parity of what was just timed, on a sample of rows (the oracle is the checker, not the thing measured)
     rows = torch.arange(0, m, 517)
@@ -164,7 +202,7 @@ def main():
         "config": {"workload": "C2: bf16 GEMM M=N=K=8192, A,B ~ N(0,1)/sqrt(K) seed 2, row-major, fp32 acc, bf16 out",
                    "tile": cfg},
         "pct_of_peak": round(100 * value / PEAK["bf16"], 2),
-        "roofline": roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "cpu_baseline": cpu, "vendor_blas": vendor,
         "parity": {"ok": bool(ok), "max_abs_err": maxerr, "max_err_over_max_ref": rel, "rows_checked": int(rows.numel())},
     }
     del a, b, c
@@ -183,7 +221,7 @@ def extras(torch, dev, oracle, mm, sg, args):
     reps = 30
 
     def measure(name, fn, flops, bytes_, dt, bound, nrot=1):
-        for i in range(5):
+        for i in range(PRE_ROLL):
             fn(i % nrot)
         torch.cuda.synchronize()
         durs = event_times(lambda i: fn(i % nrot), reps)
@@ -203,7 +241,16 @@ def extras(torch, dev, oracle, mm, sg, args):
     cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
     c = torch.empty((1024, 768), device=dev, dtype=torch.float16)
     l1 = mm.matmul_kernel.prepare(a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg)
-    measure("C1", lambda i: l1(), 805306368, 3407872, "f16", None)["tile"] = cfg
+    r = measure("C1", lambda i: l1(), 805306368, 3407872, "f16", None)
+    r["tile"] = cfg
+    if not args.no_vendor:
+        cv = torch.empty_like(c)
+        r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, b, out=cv))
+    if not args.no_cpu:
+        af, bf = a.cpu().float(), b.cpu().float()
+        t, n = cpu_time(lambda: torch.matmul(af, bf))
+        r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(805306368 / t / 1e9, 1), "cores": torch.get_num_threads(),
+                    "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
 
     # C3: B is streamed from HBM: rotate distinct copies of B so that none is served from the 256 MiB Infinity Cache
     a_cpu, b_cpu = oracle.make_inputs("C3")
@@ -219,6 +266,15 @@ def extras(torch, dev, oracle, mm, sg, args):
     r["note"] = f"{nrot} distinct copies of B rotated ({nrot * 117} MB > 256 MB Infinity Cache); one kernel, reduction fused"
     ok, _, rel = oracle.within_tolerance(c, oracle.reference_matmul(a_cpu, b_cpu))
     r["parity_ok"] = bool(ok)
+    if not args.no_vendor:
+        cv = torch.empty_like(c)
+        r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, bs[i % nrot], out=cv), reps=reps)
+    if not args.no_cpu:
+        af, bf = a_cpu.float(), b_cpu.float()
+        t, n = cpu_time(lambda: torch.matmul(af, bf))
+        r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(1879048192 / t / 1e9, 1), "cores": torch.get_num_threads(),
+                    "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
+        del af, bf
     del bs
 
     # C4: fused GLU, both activations
@@ -232,6 +288,21 @@ def extras(torch, dev, oracle, mm, sg, args):
     rows = torch.arange(0, 4096, 409)
     res["C4_sigmoid"]["parity_ok"] = bool(oracle.within_tolerance(z[rows.to(dev)],
                                                                   oracle.reference_glu(x_cpu[rows], w_cpu, "sigmoid"))[0])
+    if not args.no_vendor:
+        g1 = torch.empty((4096, 28672), device=dev, dtype=torch.bfloat16)
+        res["C4_silu"]["vendor_ms"] = vendor_ms(lambda i: torch.matmul(x, w, out=g1))
+        res["C4_silu"]["vendor_note"] = "the [4096,28672] GEMM alone; gating would be a second pass over its output"
+        del g1
+    if not args.no_cpu:
+        import torch.nn.functional as F
+
+        nr = 256
+        xf, w1, w2 = x_cpu[:nr].float(), w_cpu[:, 0::2].float(), w_cpu[:, 1::2].float()
+        t, n = cpu_time(lambda: F.silu(xf @ w1) * (xf @ w2))
+        res["C4_silu"]["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(962072674304 * nr / 4096 / t / 1e9, 1),
+                                 "cores": torch.get_num_threads(),
+                                 "sample": f"torch fp32 CPU silu(x@W1)*(x@W2), first {nr} of 4096 rows, median of {n}"}
+        del xf, w1, w2
     del x, w, z
 
     # C5: int8 -> int32
@@ -244,6 +315,19 @@ def extras(torch, dev, oracle, mm, sg, args):
     r["tile"] = cfg
     rows = torch.arange(0, 8192, 1021)
     r["bit_exact"] = bool(torch.equal(c[rows.to(dev)].cpu(), oracle.reference_matmul(a_cpu[rows], b_cpu)))
+    if not args.no_vendor and hasattr(torch, "_int_mm"):
+        try:
+            r["vendor_ms"] = vendor_ms(lambda i: torch._int_mm(a, b))
+        except Exception as e:                      # the vendor path is optional; its absence is not an error here
+            r["vendor_ms"] = None
+            r["vendor_note"] = f"torch._int_mm unavailable: {type(e).__name__}"
+    if not args.no_cpu:
+        nr = 256
+        ad, bd = a_cpu[:nr].double(), b_cpu.double()
+        t, n = cpu_time(lambda: torch.matmul(ad, bd))
+        r["cpu"] = {"ms": round(t * 1e3, 3), "gops": round(1099511627776 * nr / 8192 / t / 1e9, 1),
+                    "cores": torch.get_num_threads(),
+                    "sample": f"torch fp64 CPU matmul (exact for int8), first {nr} of 8192 rows, median of {n}"}
     return res
 
 
