@@ -59,6 +59,19 @@ def event_times(fn, n):
     return [s.elapsed_time(e) for s, e in zip(starts, stops)]
 
 
+def region_time(fn, n):
+    """Mean launch duration in ms: one HIP-event pair around n back-to-back launches on the launch stream."""
+    import torch
+
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(n):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n
+
+
 def cpu_time(fn, budget_s=8.0, max_reps=3):
     """Median wall time of fn() on the host: one warm-up, then up to max_reps timed runs inside the budget."""
     fn()
@@ -74,11 +87,10 @@ def vendor_ms(fn, reps=20):
     """Mean per-launch ms of a torch GPU op (the vendor BLAS), same event protocol as the kernels under test."""
     import torch
 
-    for _ in range(PRE_ROLL):
-        fn(0)
+    for i in range(PRE_ROLL):
+        fn(i)
     torch.cuda.synchronize()
-    durs = event_times(fn, reps)
-    return round(sum(durs) / len(durs), 4)
+    return round(region_time(fn, 2 * reps), 4)
 
 
 def pick_config(kernel, launcher, a, b, tune, split=False):
@@ -156,12 +168,14 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     value = flops * args.steps / wall / 1e12
 
-    durs = event_times(step, max(10, min(args.steps, 100)))
-    kern_ms = sum(durs) / len(durs)
+    nev = max(10, min(args.steps, 100))
+    durs = event_times(step, nev)                    # one event pair per launch: spread of single launches
+    kern_ms = region_time(step, nev)                 # one event pair around the region: mean launch duration
     achieved = flops / kern_ms / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK["bf16"], "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK["bf16"], 4), "traffic": TRAFFIC_BYTES_C2,
-                "kernel_ms": round(kern_ms, 4), "kernel_ms_min": round(min(durs), 4)}
+                "kernel_ms": round(kern_ms, 4), "kernel_ms_single_mean": round(sum(durs) / len(durs), 4),
+                "kernel_ms_single_min": round(min(durs), 4)}
 
     vendor = None
     if not args.no_vendor:
@@ -225,8 +239,8 @@ def extras(torch, dev, oracle, mm, sg, args):
             fn(i % nrot)
         torch.cuda.synchronize()
         durs = event_times(lambda i: fn(i % nrot), reps)
-        ms = sum(durs) / len(durs)
-        r = {"kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "gbs": round(bytes_ / ms / 1e6, 1)}
+        ms = region_time(lambda i: fn(i % nrot), 2 * reps)
+        r = {"kernel_ms": round(ms, 4), "kernel_ms_single_mean": round(sum(durs) / len(durs), 4), "tflops": round(flops / ms / 1e9, 2), "gbs": round(bytes_ / ms / 1e6, 1)}
         if bound == "mfma":
             r["roofline"] = {"bound": "mfma", "achieved": r["tflops"], "peak": PEAK[dt], "unit": "TFLOP/s",
                              "frac": round(r["tflops"] / PEAK[dt], 4)}

@@ -154,6 +154,7 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.ktiles_per_split = (kt_total + a->split_k - 1) / a->split_k;
   p.epilogue = a->epilogue;
   p.out_dtype = a->out_dtype;
+  p.b_once = p.tiles_m == 1;
   p.c_vec_ok = a->stride_cn == 1 && ((a->stride_cm * es_out) % 16) == 0 && (((uintptr_t)a->c) % 16) == 0;
 
   hipStream_t stream = (hipStream_t)a->stream;

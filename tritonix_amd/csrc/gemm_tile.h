@@ -52,6 +52,7 @@ struct GemmParams {
   int epilogue;
   int out_dtype;
   bool c_vec_ok;          // C takes 16-byte stores along n (stride_cn == 1, 16-byte aligned rows)
+  bool b_once;            // every element of B is read by exactly one workgroup (one tile row): stream it non-temporally
 };
 
 // ---------------------------------------------------------------------------
@@ -130,6 +131,14 @@ __host__ __device__ inline void swizzle2d(int i, int j, int size_i, int size_j, 
 // lds_base + lane*16 (lds_base wave-uniform, carried in M0).
 __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base), "v"(voff), "s"(sbase)
+               : "memory");
+}
+
+// same, with the non-temporal hint: for an operand that is streamed from HBM once and never reused
+__device__ __forceinline__ void dma16_nt(const uint8_t* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
                : "memory");
@@ -560,7 +569,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     if (q < C::A_LPW) {
       dma16(a_sbase, a_voff[q], stage_base + (q * NW + wave) * 1024);
     } else {
-      dma16(b_sbase, b_voff[q - C::A_LPW], stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
+      // short tiles are the ones used on skinny problems, where B is the HBM stream
+      if (BM <= 64 && p.b_once)
+        dma16_nt(b_sbase, b_voff[q - C::A_LPW], stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
+      else
+        dma16(b_sbase, b_voff[q - C::A_LPW], stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
     }
   };
   auto dma_advance = [&]() {
