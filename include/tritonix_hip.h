@@ -79,15 +79,24 @@ typedef struct tnx_gemm_args {
   int32_t num_stages; /* LDS ring depth of the global->LDS pipeline              */
   int32_t num_warps;  /* wavefronts (64 lanes) per workgroup: 4 or 8             */
   int32_t epilogue;   /* tnx_epilogue                                            */
+  int32_t tail_tiles; /* with split_k > 1: 0 = every tile is cut; t > 0 = see below    */
+  int32_t reserved0;  /* must be 0                                               */
   void* workspace;    /* device scratch for split_k > 1 (see tnx_gemm_workspace_bytes) */
   size_t workspace_bytes;
   void* stream;       /* hipStream_t; NULL = the null stream                     */
 } tnx_gemm_args;
 
+/* tail_tiles: with split_k > 1 and tail_tiles = t > 0 only the last t tiles in launch order
+ * are cut along K, the tiles before them are computed whole by one workgroup each.  This
+ * fills the last, partial wave of workgroups when the tile count is not a multiple of the
+ * CU count (the reference's answer to the same problem is a persistent kernel,
+ * playground/persistent_mma.py:47-141). */
+
 /* Launch one GEMM.  Returns a tnx_status.  Asynchronous. */
 int tnx_gemm(const tnx_gemm_args* args);
 
-/* Bytes of device scratch tnx_gemm needs for these args (0 when split_k <= 1).
+/* Bytes of device scratch tnx_gemm needs for these args (0 when split_k <= 1):
+ * the counters plus split_k fp32/int32 copies of every tile that is cut.
  * The workspace must be 256-byte aligned.  Its first TNX_WS_COUNTER_BYTES hold
  * per-tile arrival counters: they must be zero before the first launch that
  * uses the workspace, and every launch leaves them zero again, so one

@@ -47,7 +47,7 @@ def test_struct_layout_matches_the_header_field_order():
         decl = re.sub(r"^(const\s+)?(void|int64_t|int32_t|size_t)\s*\*?", "", decl)
         names += [n.strip(" *") for n in decl.split(",")]
     assert names == [f[0] for f in _C.GemmArgs._fields_]
-    assert ctypes.sizeof(_C.GemmArgs) == 3 * 8 + 9 * 8 + 10 * 4 + 8 + 8 + 8
+    assert ctypes.sizeof(_C.GemmArgs) == 3 * 8 + 9 * 8 + 12 * 4 + 8 + 8 + 8
 
 
 def test_lds_bytes_is_host_arithmetic():
@@ -95,7 +95,13 @@ def test_ragged_layouts_need_a_generic_kernel():
 def test_workspace_bytes_and_default_config():
     lib = _C.load()
     assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args())) == 0
-    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=16, n=4096, k=14336, split_k=8))) == 65536 + 8 * 16 * 4096 * 4
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=16, n=4096, k=14336, split_k=8))) == 65536 + 8 * 32 * 128 * 128 * 4  # 32 tiles of 128x128, eight slices each
+    # only the last 10 of the 6 x 6 tiles are cut: the workspace holds their slices and nothing else
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=768, n=768, split_k=4, tail_tiles=10))) == \
+        65536 + 4 * 10 * 128 * 128 * 4
+    assert lib.tnx_gemm_workspace_bytes(ctypes.byref(args(m=768, n=768, split_k=4, tail_tiles=99))) == \
+        65536 + 4 * 36 * 128 * 128 * 4
+    assert lib.tnx_gemm_supported(ctypes.byref(args(tail_tiles=-1))) == _C.E_INVALID
     g = args(m=8192, n=8192, k=8192)
     assert lib.tnx_gemm_default_config(ctypes.byref(g)) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK

@@ -226,6 +226,43 @@ def test_error_mapping_on_launch(device):
         gemm(a.cpu(), a.cpu(), GENERIC)
 
 
+# ---- K cut only for the trailing tiles (fills the last, partial wave of workgroups) ------
+@pytest.mark.parametrize("tail,split_k", [(1, 2), (5, 4), (16, 4), (47, 8), (48, 2), (200, 4)])
+def test_tail_tiles_split_bf16(device, tail, split_k):
+    g = torch.Generator("cpu").manual_seed(tail * 100 + split_k)
+    a = (torch.randn(700, 2048, generator=g) / 45.0).to(torch.bfloat16)      # 6 x 8 = 48 tiles of 128x128, ragged M
+    b = torch.randn(2048, 1000, generator=g).to(torch.bfloat16)
+    ref = oracle.reference_matmul(a, b)
+    ad, bd = a.to(device), b.to(device)
+    config = cfg(128, 128, 64, 4, 3, split_k=split_k, tail_tiles=tail)
+    out = gemm(ad, bd, config, kernel=gemm_splitk_kernel)
+    check_fp(out, ref)
+    assert torch.equal(gemm(ad, bd, config, kernel=gemm_splitk_kernel), out)          # slices are added in slice order
+    # whole tiles of the same launch are bit-identical to the plain kernel's
+    plain = gemm(ad, bd, cfg(128, 128, 64, 4, 3))
+    assert (out == plain).float().mean() > (48 - min(tail, 48)) / 48 - 1e-6
+    # matmul_kernel takes the same two keywords
+    assert torch.equal(gemm(ad, bd, config, kernel=matmul_kernel), out)
+
+
+def test_tail_tiles_int8_exact_and_glu(device):
+    g = torch.Generator("cpu").manual_seed(77)
+    a = torch.randint(-127, 128, (520, 1024), generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (1024, 768), generator=g, dtype=torch.int8)
+    out = gemm(a.to(device), b.to(device), cfg(128, 128, 128, 4, 2, split_k=4, tail_tiles=7), kernel=gemm_splitk_kernel)
+    assert torch.equal(out.cpu(), oracle.reference_matmul(a, b))
+    out = gemm(a.to(device), b.to(device), cfg(256, 256, 128, 4, 2, split_k=3), kernel=gemm_splitk_kernel)
+    assert torch.equal(out.cpu(), oracle.reference_matmul(a, b))
+    # gated epilogue on a launch whose last tiles are cut
+    x = (torch.randn(300, 1024, generator=g)).to(torch.bfloat16)
+    w = (0.05 * torch.randn(1024, 1536, generator=g)).to(torch.bfloat16)
+    xd, wd = x.to(device), w.to(device)
+    for act in ("silu", "sigmoid"):
+        z = torch.full((300, 768), 7, device=device, dtype=torch.bfloat16)
+        run(glu_kernel, xd, wd, z, cfg(128, 128, 64, 4, 2), use_tf32=True, activation=act, split_k=4, tail_tiles=11)
+        check_fp(z, oracle.reference_glu(x, w, act))
+
+
 # ---- wavefront-level split-K kernel (m <= 16, eight K slices meet in LDS) ---------------
 @pytest.mark.parametrize("m,n,k,stages,dtype", [(16, 4096, 14336, 6, torch.bfloat16), (16, 512, 2048, 3, torch.bfloat16),
                                                 (5, 96, 512, 4, torch.bfloat16), (1, 32, 256, 5, torch.float16)])

@@ -38,7 +38,7 @@ class GemmArgs(ctypes.Structure):
         ("block_m", ctypes.c_int32), ("block_n", ctypes.c_int32), ("block_k", ctypes.c_int32),
         ("group_m", ctypes.c_int32), ("split_k", ctypes.c_int32),
         ("num_stages", ctypes.c_int32), ("num_warps", ctypes.c_int32),
-        ("epilogue", ctypes.c_int32),
+        ("epilogue", ctypes.c_int32), ("tail_tiles", ctypes.c_int32), ("reserved0", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
     ]

@@ -48,7 +48,7 @@ static int check_common(const tnx_gemm_args* a) {
   if (a->in_dtype != TNX_F16 && a->in_dtype != TNX_BF16 && a->in_dtype != TNX_I8) return TNX_E_INVALID;
   if (a->epilogue < TNX_EPI_NONE || a->epilogue > TNX_EPI_GLU_IDENTITY) return TNX_E_INVALID;
   if (a->block_m <= 0 || a->block_n <= 0 || a->block_k <= 0 || a->group_m <= 0 || a->split_k <= 0 ||
-      a->num_stages <= 0 || a->num_warps <= 0)
+      a->num_stages <= 0 || a->num_warps <= 0 || a->tail_tiles < 0 || a->reserved0 != 0)
     return TNX_E_INVALID;
   // output type is tied to the input type: f16->f16, bf16->bf16, i8->i32
   int want_out = a->in_dtype == TNX_I8 ? TNX_I32 : a->in_dtype;
@@ -78,10 +78,19 @@ extern "C" int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* a) {
   return lds_bytes_of(a);
 }
 
+// tiles that are cut along K: all of them, or the last tail_tiles in launch order
+static int64_t cut_tiles(const tnx_gemm_args* a) {
+  if (a->block_m <= 0 || a->block_n <= 0) return 0;
+  int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
+  if (a->split_k <= 1) return 0;
+  return a->tail_tiles > 0 && a->tail_tiles < tiles ? a->tail_tiles : tiles;
+}
+
 extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
   if (!a || a->split_k <= 1 || a->m <= 0 || a->n <= 0) return 0;
   if (is_skinny_cfg(a)) return 0;   // the eight K slices meet in LDS
-  return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)a->m * (size_t)a->n * 4;
+  // every slice of a cut tile is kept whole (block_m x block_n accumulators of 4 bytes)
+  return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)cut_tiles(a) * (size_t)a->block_m * (size_t)a->block_n * 4;
 }
 
 static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs) {
@@ -113,7 +122,7 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   if (!f && !e->generic) return TNX_E_UNSUPPORTED;
   int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
   if (tiles * a->split_k > 0x7fffffffll) return TNX_E_UNSUPPORTED;
-  if (a->split_k > 1 && tiles > WS_MAX_TILES) return TNX_E_UNSUPPORTED;  // one arrival counter per tile
+  if (cut_tiles(a) > WS_MAX_TILES) return TNX_E_UNSUPPORTED;  // one arrival counter per cut tile
   if (out) *out = e;
   if (fast) *fast = f;
   return TNX_OK;
@@ -150,6 +159,8 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.tiles_n = (int)((a->n + a->block_n - 1) / a->block_n);
   p.group_m = a->group_m;
   p.split_k = a->split_k;
+  const int64_t ncut = cut_tiles(a);
+  p.split_tile0 = a->split_k > 1 ? (int)((int64_t)p.tiles_m * p.tiles_n - ncut) : 0;
   int kt_total = (int)((a->k + a->block_k - 1) / a->block_k);
   p.ktiles_per_split = (kt_total + a->split_k - 1) / a->split_k;
   p.epilogue = a->epilogue;
@@ -162,7 +173,7 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   if (is_skinny_cfg(a)) {
     err = skinny_lookup(a->in_dtype, a->num_stages)(p, (unsigned)(a->n / SKINNY_BN), stream);
   } else {
-    unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * a->split_k);
+    unsigned grid = a->split_k > 1 ? (unsigned)(p.split_tile0 + ncut * a->split_k) : (unsigned)(p.tiles_m * p.tiles_n);
     err = (fast ? e->fast : e->generic)(p, grid, stream);
   }
   if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
@@ -203,13 +214,30 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     a->block_m = a->m <= 64 ? 64 : 128; a->block_n = 128; a->num_stages = 2; a->num_warps = 4;
     return TNX_OK;
   }
+  // Pick the (tile, K split) pair with the smallest modelled time: waves of workgroups over 256 CUs,
+  // each tile costing its multiply-adds over the rate a CU sustains with that tile (relative rates
+  // measured on 8192^3: 256x256 1.0, 256x128 0.9, 128x128 0.7), plus a fixed cost for the split-K
+  // hand-over (partials through memory, one more round trip).  K is only cut when the tiles
+  // alone leave CUs idle, and never into pieces shorter than eight K slabs.
   static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
+  static const double rate[] = {1.0, 0.9, 0.7, 0.5, 0.35};
   const int ncand = es == 1 ? 4 : 5;   // int8 rows of a 64-wide B tile are too short for the transposing read
+  const double cu_flops = 5.5e12 * (es == 1 ? 1.7 : 1.0);          // per CU with the largest tile
+  const int64_t kt = (a->k + bk - 1) / bk;
+  double best = 1e300;
+  int bi = 0, bs = 1;
   for (int i = 0; i < ncand; ++i) {
-    a->block_m = cand[i][0]; a->block_n = cand[i][1]; a->num_stages = cand[i][2]; a->num_warps = cand[i][3];
-    int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
-    if (tiles >= cus * 3 / 4) break;
+    const int64_t tiles = ((a->m + cand[i][0] - 1) / cand[i][0]) * ((a->n + cand[i][1] - 1) / cand[i][1]);
+    for (int s = 1; s <= 16; s *= 2) {
+      if (s > 1 && (tiles * s > cus + cus / 4 || kt / s < 8)) break;
+      const int64_t waves = (tiles * s + cus - 1) / cus;
+      const double t = (double)waves * (2.0 * cand[i][0] * cand[i][1] * (double)a->k / s) / (cu_flops * rate[i]) +
+                       (s > 1 ? 4e-6 : 0.0) + 3e-6;
+      if (t < best * 0.97) { best = t; bi = i; bs = s; }             // ties go to the earlier (larger, unsplit) choice
+    }
   }
+  a->block_m = cand[bi][0]; a->block_n = cand[bi][1]; a->num_stages = cand[bi][2]; a->num_warps = cand[bi][3];
+  a->split_k = bs;
   return TNX_OK;
 }
 

@@ -48,6 +48,7 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int group_m;
   int split_k;
+  int split_tile0;        // tiles [0, split_tile0) in launch order are computed whole; the rest are cut split_k ways
   int ktiles_per_split;   // K slabs handled by one split
   int epilogue;
   int out_dtype;
@@ -150,22 +151,21 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
   return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
-// Device-scope (all XCDs) 16-byte and 4-byte accesses for data that workgroups hand to each
-// other inside one kernel: the sc1 bit writes through / reads around the per-XCD L2, so no
-// whole-cache write-back or invalidate is needed around them.
+// Device-scope (all XCDs) 16-byte accesses for data that workgroups hand to each other inside
+// one kernel: the sc1 bit writes through / reads around the per-XCD L2, so no whole-cache
+// write-back or invalidate is needed around them.  The load does not wait: loads_landed()
+// does, for all loads passed to it.
 __device__ __forceinline__ void store16_agent(void* dst, i32x4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
 }
-__device__ __forceinline__ i32x4 load16_agent(const void* src) {
-  i32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(src) : "memory");
-  return v;
+__device__ __forceinline__ void load16_agent_nowait(i32x4& v, const void* src) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(src) : "memory");
 }
-__device__ __forceinline__ void store4_agent(int* dst, int v) {
-  __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ int load4_agent(const int* src) {
-  return __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+template <int N> __device__ __forceinline__ void loads_landed(i32x4 (&v)[N]) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // tie every loaded value to the wait, so that no use is scheduled above it
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i]) : : "memory");
 }
 
 template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
@@ -233,7 +233,7 @@ struct TileCfg {
   static constexpr bool VALID =
       (WTM % 16 == 0) && (WTN % 16 == 0) && (BK * ES) % KB == 0 && KSTEPS >= 1 && CPR_A >= 4 &&
       (ES == 2 ? CPR_B >= 8 : CPR_B >= 8) && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
-      LDS_BYTES <= 163840 && TM * TN * ACC_N <= 256 && (STAGES - 2) * LPW <= 63 && STAGES >= 2;
+      A_LOADS % NW == 0 && B_LOADS % NW == 0 && LDS_BYTES <= 163840 && TM * TN * ACC_N <= 256 && (STAGES - 2) * LPW <= 63 && STAGES >= 2;
 
   // chunk-index XOR applied to row `row` of the A slab
   static __host__ __device__ constexpr int swzA(int row) {
@@ -267,8 +267,6 @@ template <> struct OutOf<TagBF16> { typedef OutBF16 type; };
 template <> struct OutOf<TagF16> { typedef OutF16 type; };
 template <> struct OutOf<TagI8> { typedef int type; };
 
-template <class O, class S> struct Cvt1 { typedef typename O::raw raw; static __device__ __forceinline__ raw run(S v) { return O::cvt((float)v); } };
-template <> struct Cvt1<int, int> { typedef int raw; static __device__ __forceinline__ int run(int v) { return v; } };
 
 // LDS one wave needs to pass one row-block (MI rows) of its accumulators through LDS: raw
 // 32-bit values, rows padded by 16 bytes to spread the banks.
@@ -289,14 +287,6 @@ template <class O, bool GLU> struct Pack16<O, float, GLU> {   // 16-bit float ou
     for (int x = 0; x < OUTV; ++x) out[x] = O::cvt(GLU ? glu_gate(f[2 * x], epi) * f[2 * x + 1] : f[x]);
   }
 };
-template <bool GLU> struct Pack16<float, float, GLU> {        // fp32 outputs (split-K partials): 4 per lane
-  typedef float raw;
-  static constexpr int OUTV = 4, NF = 4;
-  static __device__ __forceinline__ void run(const float* f, int, raw* out) {
-#pragma unroll
-    for (int x = 0; x < 4; ++x) out[x] = f[x];
-  }
-};
 template <bool GLU> struct Pack16<int, int, GLU> {            // int32 outputs: 4 per lane
   typedef int raw;
   static constexpr int OUTV = 4, NF = 4;
@@ -306,17 +296,70 @@ template <bool GLU> struct Pack16<int, int, GLU> {            // int32 outputs: 
   }
 };
 
+// Where the split-K slices of one wave's part of a tile sit in the workspace.  A slice is
+// stored exactly as the wave holds it: group q = (i*TN + j)*NGRP + g of four accumulator
+// registers is one 16-byte element per lane at q*1024 + lane*16, so every store and load
+// instruction moves one contiguous KiB.
+struct SliceSrc {
+  const uint8_t* base;     // this wave's part of slice 0
+  int64_t slice_stride;    // bytes from one slice to the next
+  int nslices;
+};
+
+// Sum of the split-K slices of one row-block of a wave, group by group, into the wave's LDS
+// strip (same places the accumulators of an uncut tile go).  ZB slices of G = 32 / ZB groups
+// are fetched together; slices are added in slice order whatever ZB is.
+template <class ACC4, int ZB, int NQ, int MI, int NGRP>
+__device__ __forceinline__ void sum_slices(const uint8_t* q0, const SliceSrc& src, uint32_t wbase, bool row_ok) {
+  constexpr int G = (32 / ZB) < NQ ? (32 / ZB) : NQ;
+  static_assert(NQ % G == 0, "groups per row-block must be a multiple of the batch");
+#pragma unroll 1
+  for (int jg0 = 0; jg0 < NQ; jg0 += G) {
+    ACC4 v[G];
+#pragma unroll
+    for (int x = 0; x < G; ++x) v[x] = ACC4{0, 0, 0, 0};
+    // lanes whose row lies past the last row of the problem were not stored and are not read
+#pragma unroll 1
+    for (int z0 = 0; row_ok && z0 < src.nslices; z0 += ZB) {
+      i32x4 w[G * ZB];
+#pragma unroll
+      for (int x = 0; x < G; ++x)
+#pragma unroll
+        for (int u = 0; u < ZB; ++u) {
+          const int z = z0 + u < src.nslices ? z0 + u : src.nslices - 1;
+          load16_agent_nowait(w[x * ZB + u], q0 + (int64_t)(jg0 + x) * 1024 + z * src.slice_stride);
+        }
+      loads_landed(w);
+#pragma unroll
+      for (int x = 0; x < G; ++x)
+#pragma unroll
+        for (int u = 0; u < ZB; ++u)
+          if (z0 + u < src.nslices) {
+            ACC4 t;
+            __builtin_memcpy(&t, &w[x * ZB + u], 16);
+            v[x] += t;
+          }
+    }
+#pragma unroll
+    for (int x = 0; x < G; ++x) {
+      const int j = (jg0 + x) / NGRP, g = (jg0 + x) % NGRP;
+      *TNX_LDS(ACC4, wbase + (j * MI + g * 8) * 4) = v[x];
+    }
+  }
+}
+
 // The MFMA result is C^T: lane l owns output row m = l % MI and, per group of four accumulator
 // registers, four consecutive columns n.  Each wave passes one row-block at a time through its
-// private LDS strip: raw accumulators in (one ds_write_b128 per group, nothing else in the
-// unrolled part), then a plain loop reads the strip row-major, converts / gates, and stores 16
-// bytes per lane, so every row of C receives full contiguous runs.  Keeping the conversion out
-// of the unrolled part keeps the three epilogue variants of a 256x256 tile inside the
-// instruction cache.
-template <class T, class C, class O, bool GLU, bool AGENT, class ACC>
-__device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t lds_strip, int lane,
-                                               int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
-                                               int64_t scn, bool vec_ok, int epi) {
+// private LDS strip: raw accumulators in (one ds_write_b128 per group), then a plain loop reads
+// the strip row-major, converts / gates, and stores 16 bytes per lane, so every row of C
+// receives full contiguous runs.  Keeping the conversion out of the unrolled part keeps the
+// epilogue variants of a 256x256 tile inside the instruction cache.
+// FROM_WS: the values do not come from this wave's registers but from the split-K slices in
+// the workspace, added in slice order (the result does not depend on which workgroup does it).
+template <class T, class C, class O, bool GLU, bool FROM_WS, class ACC>
+__device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const SliceSrc& src, uint8_t* cbase,
+                                               uint32_t lds_strip, int lane, int64_t gm0, int64_t gc0, int64_t m,
+                                               int64_t ncols, int64_t scm, int64_t scn, bool vec_ok, int epi) {
   typedef typename T::acc_s acc_s;
   typedef Pack16<O, acc_s, GLU> PK;
   typedef typename PK::raw raw;
@@ -327,48 +370,69 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t
   constexpr int WCOLS = GLU ? C::WTN / 2 : C::WTN;      // output columns of the wave tile
   constexpr int CPRW = WCOLS / PK::OUTV;                // 16-byte output chunks per strip row
   constexpr int ITERS = (MI * CPRW + 63) / 64;
+  constexpr int UNR = ITERS % 4 == 0 ? 4 : (ITERS % 2 == 0 ? 2 : 1);   // read-back rows in flight together
   static_assert(WCOLS % PK::OUTV == 0, "wave tile too narrow for 16-byte stores");
   raw* cp = (raw*)cbase;
   const uint32_t wbase = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
+    if (gm0 + i * MI >= m) break;                       // row-blocks past the last row hold nothing
+    if constexpr (!FROM_WS) {
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j)
+      for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-      for (int g = 0; g < NGRP; ++g)
-        // (typed vector store: __builtin_bit_cast on an ext-vector element reads element 0)
-        *TNX_LDS(acc4, wbase + (j * MI + g * 8) * 4) =
-            acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        for (int g = 0; g < NGRP; ++g)
+          // (typed vector store: __builtin_bit_cast on an ext-vector element reads element 0)
+          *TNX_LDS(acc4, wbase + (j * MI + g * 8) * 4) =
+              acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+    } else {
+      // 32 loads per lane in flight (G groups x ZB slices): the hand-over is latency-bound otherwise
+      const uint8_t* q0 = src.base + (int64_t)i * (C::TN * NGRP) * 1024 + lane * 16;
+      const bool row_ok = gm0 + i * MI + lane % MI < m;
+      if (src.nslices <= 2)
+        sum_slices<acc4, 2, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+      else if (src.nslices <= 4)
+        sum_slices<acc4, 4, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+      else
+        sum_slices<acc4, 8, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+    }
     // the strip is private to this wave: its own LDS writes are ordered before its reads
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
 #pragma unroll 1
-    for (int it = 0; it < ITERS; ++it) {
-      const int q = it * 64 + lane;
-      const int row = q / CPRW, cc = q % CPRW;
-      const int64_t gm = gm0 + i * MI + row;
-      const int64_t gc = gc0 + cc * PK::OUTV;
-      if ((MI * CPRW % 64 != 0 && row >= MI) || gm >= m) continue;
-      acc_s f[PK::NF];
+    for (int it0 = 0; it0 < ITERS; it0 += UNR) {
+      // UNR rows of LDS reads are issued together, then converted and stored one after the other
+      acc_s f[UNR][PK::NF];
 #pragma unroll
-      for (int x = 0; x < PK::NF / 4; ++x) {
-        const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * PK::NF + 4 * x) * 4);
-        __builtin_memcpy(&f[4 * x], &v, 16);
+      for (int u = 0; u < UNR; ++u) {
+        const int q = (it0 + u) * 64 + lane;
+        int row = q / CPRW;
+        const int cc = q % CPRW;
+        if (MI * CPRW % 64 != 0 && row >= MI) row = MI - 1;
+#pragma unroll
+        for (int x = 0; x < PK::NF / 4; ++x) {
+          const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * PK::NF + 4 * x) * 4);
+          __builtin_memcpy(&f[u][4 * x], &v, 16);
+        }
       }
-      raw out[PK::OUTV];
-      PK::run(f, epi, out);
-      raw* dst = cp + gm * scm + gc * scn;
-      if (vec_ok && gc + PK::OUTV <= ncols) {
-        i32x4 v;
-        __builtin_memcpy(&v, out, 16);
-        if constexpr (AGENT) store16_agent(dst, v);
-        else *(i32x4*)dst = v;
-      } else {
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int q = (it0 + u) * 64 + lane;
+        const int row = q / CPRW, cc = q % CPRW;
+        const int64_t gm = gm0 + i * MI + row;
+        const int64_t gc = gc0 + cc * PK::OUTV;
+        if ((MI * CPRW % 64 != 0 && row >= MI) || gm >= m) continue;
+        raw out[PK::OUTV];
+        PK::run(f[u], epi, out);
+        raw* dst = cp + gm * scm + gc * scn;
+        if (vec_ok && gc + PK::OUTV <= ncols) {
+          i32x4 v;
+          __builtin_memcpy(&v, out, 16);
+          *(i32x4*)dst = v;
+        } else {
 #pragma unroll 1
-        for (int x = 0; x < PK::OUTV; ++x)
-          if (gc + x < ncols) {
-            if constexpr (AGENT) store4_agent((int*)dst + x * scn, __builtin_bit_cast(int, out[x]));
-            else dst[x * scn] = out[x];
-          }
+          for (int x = 0; x < PK::OUTV; ++x)
+            if (gc + x < ncols) dst[x * scn] = out[x];
+        }
       }
     }
     // the next row-block overwrites the strip: wait for the reads above
@@ -376,89 +440,57 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], uint8_t
   }
 }
 
-// The first WS_COUNTER_BYTES of the split-K workspace hold one arrival counter per output
-// tile.  They must be zero when a launch starts; every launch leaves them zero.
+// The first WS_COUNTER_BYTES of the split-K workspace hold one arrival counter per cut tile.
+// They must be zero when a launch starts; every launch leaves them zero.
 constexpr int WS_COUNTER_BYTES = 65536;
 constexpr int WS_MAX_TILES = WS_COUNTER_BYTES / 4;
 
-// Split-K tail.  Every wave has just stored its partial with device-scope stores.  One lane
-// bumps the tile's counter, and the workgroup that finds the counter at split_k-1 owns the
-// reduction: it reads the slices back with device-scope loads, adds them in slice order (so
-// the result does not depend on arrival order), applies the epilogue, writes C and re-arms
-// the counter.  Whole-L2 write-backs and invalidates (what a device-scope fence costs on a
-// part with eight L2s) are avoided on purpose: they cost more than the GEMM.
-template <class T, class C>
-__device__ __forceinline__ void splitk_finish(const GemmParams& p, const typename T::acc_s* part, int* counter, int* flag,
-                                              int64_t m0, int64_t n0) {
+// One K slice of a cut tile leaves the workgroup: every wave writes its accumulators to its
+// part of the slice with device-scope (sc1) stores, one lane bumps the tile's arrival counter,
+// and the function returns true in the workgroup that arrived last.  That workgroup then reads
+// all slices back with device-scope loads and runs the ordinary epilogue on their sum.
+// Whole-L2 write-backs and invalidates (what a device-scope fence costs on a part with eight
+// L2s) are avoided on purpose: they cost more than the GEMM.
+template <class T, class C, class ACC>
+__device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t* wave_slice, uint32_t lds_strip, int lane,
+                                              int64_t gm0, int64_t m, int* counter, int* flag, int nslices) {
   typedef typename T::acc_s acc_s;
-  typedef typename OutOf<T>::type O;
-  typedef Cvt1<O, acc_s> CV;
-  typedef typename CV::raw raw;
-  // the partial was written with device-scope stores: once this wave's stores are acknowledged
-  // they are visible to every XCD, so the arrival count may follow
+  typedef acc_s acc4 __attribute__((ext_vector_type(4)));
+  constexpr int NGRP = C::ACC_N / 4;
+  constexpr int NQ = C::TN * NGRP;                      // 16-byte groups per lane and row-block
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+    if (gm0 + i * C::MI >= m) break;
+    // registers -> LDS -> registers keeps the copy loop rolled (the accumulators may sit in AGPRs,
+    // which a 16-byte device-scope store cannot name directly)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int g = 0; g < NGRP; ++g)
+        *TNX_LDS(acc4, lds_strip + (j * NGRP + g) * 1024 + lane * 16) =
+            acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    uint8_t* dst = wave_slice + (int64_t)i * NQ * 1024 + lane * 16;
+    if (gm0 + i * C::MI + lane % C::MI < m) {            // a lane is one row: rows past the problem are not stored
+#pragma unroll 4
+      for (int q = 0; q < NQ; ++q) store16_agent(dst + q * 1024, *TNX_LDS(i32x4, lds_strip + q * 1024 + lane * 16));
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+  }
+  // device-scope stores: once they are acknowledged they are visible to every XCD, so the
+  // arrival count may follow
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  if (*flag != p.split_k - 1) return;
-  const bool vec_in = (p.n & 3) == 0;
-  const bool glu = p.epilogue != EPI_NONE;
-  raw* cp = (raw*)p.c;
-  for (int idx = threadIdx.x; idx < C::BM * (C::BN / 4); idx += C::THREADS) {
-    const int row = idx / (C::BN / 4), c4 = idx % (C::BN / 4);
-    const int64_t gm = m0 + row, gn = n0 + c4 * 4;
-    if (gm >= p.m || gn >= p.n) continue;
-    acc_s v[4] = {0, 0, 0, 0};
-    // slices are fetched eight at a time (all loads in flight together), then added in slice order
-    for (int z0 = 0; z0 < p.split_k; z0 += 8) {
-      acc_s q[8][4];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int z = z0 + u < p.split_k ? z0 + u : p.split_k - 1;
-        const acc_s* src = part + ((int64_t)z * p.m + gm) * p.n + gn;
-        if (vec_in) {
-          const uint64_t lo = __hip_atomic_load((const uint64_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint64_t hi = __hip_atomic_load((const uint64_t*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          q[u][0] = __builtin_bit_cast(acc_s, (uint32_t)lo); q[u][1] = __builtin_bit_cast(acc_s, (uint32_t)(lo >> 32));
-          q[u][2] = __builtin_bit_cast(acc_s, (uint32_t)hi); q[u][3] = __builtin_bit_cast(acc_s, (uint32_t)(hi >> 32));
-        } else {
-#pragma unroll
-          for (int x = 0; x < 4; ++x)
-            q[u][x] = gn + x < p.n ? __builtin_bit_cast(acc_s, load4_agent((const int*)src + x)) : (acc_s)0;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (z0 + u < p.split_k) { v[0] += q[u][0]; v[1] += q[u][1]; v[2] += q[u][2]; v[3] += q[u][3]; }
-    }
-    if (glu) {
-      const int64_t nh = p.n >> 1, gc = gn >> 1;
-      raw* dst = cp + gm * p.scm + gc * p.scn;
-      raw z0 = CV::run((acc_s)(glu_gate((float)v[0], p.epilogue) * (float)v[1]));
-      raw z1 = CV::run((acc_s)(glu_gate((float)v[2], p.epilogue) * (float)v[3]));
-      if (gc < nh) dst[0] = z0;
-      if (gc + 1 < nh) dst[p.scn] = z1;
-    } else {
-      raw* dst = cp + gm * p.scm + gn * p.scn;
-      if (p.c_vec_ok && gn + 3 < p.n) {
-        raw r[4] = {CV::run(v[0]), CV::run(v[1]), CV::run(v[2]), CV::run(v[3])};
-        if constexpr (sizeof(raw) == 2) {
-          i32x2 pk;
-          __builtin_memcpy(&pk, r, 8);
-          *(i32x2*)dst = pk;
-        } else {
-          i32x4 pk;
-          __builtin_memcpy(&pk, r, 16);
-          *(i32x4*)dst = pk;
-        }
-      } else {
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-          if (gn + x < p.n) dst[x * p.scn] = CV::run(v[x]);
-      }
-    }
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the last arrival re-arms the counter for the next launch
+    if (prev == nslices - 1) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = prev;
   }
-  if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const bool last = *flag == nslices - 1;
+  __syncthreads();                                      // the flag's LDS word is reused by the epilogue strips
+  return last;
 }
 
 template <bool B> struct BoolTag { static constexpr bool value = B; };
@@ -470,6 +502,7 @@ template <class T, class C, bool FAST>
 __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
   constexpr int MI = C::MI, TM = C::TM, TN = C::TN;
+  static_assert(C::VALID, "tile configuration not supported by this kernel");
   typedef Mma<T, MI> MMA;
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
@@ -483,18 +516,29 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   // ---- which tile / split ------------------------------------------------
+  // Tiles [0, split_tile0) in launch order are computed whole by one workgroup each; the
+  // tiles after them are cut split_k ways along K (all tiles when split_tile0 == 0: plain
+  // split-K; only the last partial wave of tiles when the tile count does not fill the CUs).
   const int ntiles = p.tiles_m * p.tiles_n;
-  int bid = blockIdx.x;
-  const int split = bid / ntiles;
-  bid -= split * ntiles;
-  const int logical = xcd_remap(bid, ntiles, 8);
+  int split = 0, logical;
+  bool cut = false;
+  if ((int)blockIdx.x < p.split_tile0) {
+    logical = xcd_remap(blockIdx.x, p.split_tile0, 8);
+  } else {
+    const int ncut = ntiles - p.split_tile0;
+    int t = blockIdx.x - p.split_tile0;
+    split = t / ncut;
+    t -= split * ncut;
+    logical = p.split_tile0 + xcd_remap(t, ncut, 8);
+    cut = p.split_k > 1;
+  }
   int pid_m, pid_n;
   swizzle2d(logical / p.tiles_n, logical % p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, &pid_m, &pid_n);
   const int64_t m0 = (int64_t)pid_m * BM, n0 = (int64_t)pid_n * BN;
 
   const int kt_total = (int)((p.k + BK - 1) / BK);
-  const int kt0 = split * p.ktiles_per_split;
-  int kt1 = kt0 + p.ktiles_per_split;
+  const int kt0 = cut ? split * p.ktiles_per_split : 0;
+  int kt1 = cut ? kt0 + p.ktiles_per_split : kt_total;
   if (kt1 > kt_total) kt1 = kt_total;
   const int KT = kt1 > kt0 ? kt1 - kt0 : 0;          // slabs of this workgroup
   // FAST kernels are only launched when k % BK == 0 and A, B are row-major
@@ -786,21 +830,28 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int64_t gm0 = m0 + wy * C::WTM;
   const int64_t gn0 = n0 + wx * C::WTN;
   const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
-  if (p.split_k > 1) {
-    // fp32 / int32 partial of this K slice -> workspace [split][m][n]; the workgroup that
-    // arrives last at the tile's counter sums all slices in slice order and writes C
-    acc_s* part = (acc_s*)(p.ws + WS_COUNTER_BYTES);
-    epilogue_store<T, C, acc_s, false, true>(acc, (uint8_t*)(part + (int64_t)split * p.m * p.n), strip, lane, gm0, gn0, p.m,
-                                             p.n, p.n, 1, (p.n & 3) == 0, 0);
-    splitk_finish<T, C>(p, part, (int*)p.ws + logical, (int*)smem, m0, n0);
-    return;
-  } else {
-    typedef typename OutOf<T>::type O;
+  typedef typename OutOf<T>::type O;
+  if (cut) {
+    // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
+    const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;
+    const int64_t slice_stride = (int64_t)ncut * BM * BN * 4;
+    uint8_t* wave0 = p.ws + WS_COUNTER_BYTES + ((int64_t)ctile * NW + wave) * (C::WTM * C::WTN * 4);
+    if (!splitk_arrive<T, C>(acc, wave0 + split * slice_stride, strip, lane, gm0, p.m, (int*)p.ws + ctile, (int*)smem,
+                             p.split_k))
+      return;
+    const SliceSrc src = {wave0, slice_stride, p.split_k};
     if (p.epilogue == EPI_NONE)
-      epilogue_store<T, C, O, false, false>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+      epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
     else
-      epilogue_store<T, C, O, true, false>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok,
-                                           p.epilogue);
+      epilogue_store<T, C, O, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                          p.c_vec_ok, p.epilogue);
+  } else {
+    const SliceSrc none = {nullptr, 0, 0};
+    if (p.epilogue == EPI_NONE)
+      epilogue_store<T, C, O, false, false>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+    else
+      epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                           p.c_vec_ok, p.epilogue);
   }
 }
 

@@ -78,7 +78,11 @@ class HipKernel:
         self.__doc__ = doc
         self.tile_params = list(tile_params)
         self.glu = glu
-        self.arg_names = list(_POSITIONAL) + self.tile_params + (["use_tf32", "activation"] if glu else [])
+        # optional keywords after the reference's own: a K split for kernels whose signature has none, and
+        # the number of trailing tiles the split applies to (0 = all)
+        self.optional = [n for n in ("split_k", "tail_tiles") if n not in self.tile_params]
+        self.arg_names = (list(_POSITIONAL) + self.tile_params + (["use_tf32", "activation"] if glu else [])
+                          + self.optional)
         self.pre_run_hooks: List[Callable] = []
         self.specialize_keys: List[str] = []
 
@@ -121,6 +125,7 @@ class HipKernel:
         g.block_m, g.block_n, g.block_k = int(bound["block_m"]), int(bound["block_n"]), int(bound["block_k"])
         g.group_m = int(bound["group_m"])
         g.split_k = int(bound.get("split_k", 1))
+        g.tail_tiles = int(bound.get("tail_tiles", 0))
         g.num_stages, g.num_warps = int(bound["num_stages"]), int(bound["num_warps"])
         if self.glu:
             # "silu" and "sigmoid" gate explicitly; like the reference kernel, any other
