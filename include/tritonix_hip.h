@@ -116,8 +116,11 @@ int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* args);
  * otherwise the status it would return.  Pure host arithmetic. */
 int tnx_gemm_supported(const tnx_gemm_args* args);
 
-/* Fill block_m/n/k, group_m, split_k, num_stages, num_warps of `args` with a
- * built-in choice for its shape and dtype (used when nothing was tuned). */
+/* Fill block_m/n/k, group_m, split_k, tail_tiles, num_stages, num_warps of
+ * `args` with a built-in choice for its shape and dtype (used when nothing
+ * was tuned).  split_k > 1 comes back only for shapes whose tiles alone leave
+ * CUs idle; a caller that cannot provide a workspace may reset split_k to 1
+ * and tail_tiles to 0. */
 int tnx_gemm_default_config(tnx_gemm_args* args);
 
 /* Number of compiled tile kernels, and a description of the i-th one:

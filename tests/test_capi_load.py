@@ -118,3 +118,45 @@ def test_kernel_table_lists_every_dtype():
     assert len(names) == _C.load().tnx_kernel_count() > 0
     assert {n.split()[0] for n in names} == {"bf16", "f16", "i8"}
     assert _C.load().tnx_kernel_name(len(names)) is None
+
+
+def test_default_config_is_always_launchable():
+    """Whatever shape and dtype: the built-in choice names a kernel that exists, and its K cut fits one wave of CUs."""
+    lib = _C.load()
+    shapes = [(8192, 8192, 8192), (1024, 768, 512), (4096, 28672, 4096), (16, 4096, 14336), (6144, 6144, 6144),
+              (5120, 5120, 8192), (4096, 5120, 4096), (2048, 2048, 8192), (512, 2048, 8192), (512, 512, 512),
+              (128, 128, 128), (1, 8, 64), (64, 64, 64), (300, 200, 100), (4097, 4095, 4096), (256, 8192, 8192),
+              (33, 1024, 8192), (65, 12288, 4096), (10000, 10000, 1000), (2048, 2048, 64)]
+    for dt, out in ((_C.BF16, _C.BF16), (_C.F16, _C.F16), (_C.I8, _C.I32)):
+        for m, n, k in shapes:
+            g = args(m=m, n=n, k=k, stride_am=k, stride_bk=n, stride_cm=n, in_dtype=dt, out_dtype=out)
+            assert lib.tnx_gemm_default_config(ctypes.byref(g)) == _C.OK
+            assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK, (dt, m, n, k, g.block_m, g.block_n, g.block_k)
+            tiles = -(-m // g.block_m) * -(-n // g.block_n)
+            assert 1 <= g.split_k <= 16 and 0 <= g.tail_tiles < max(tiles, 1)
+            if g.split_k > 1:
+                cut = g.tail_tiles or tiles
+                assert cut * g.split_k <= 256 + (0 if m > 64 else 256)      # one wave of workgroups (skinny: up to two)
+                assert -(-k // g.block_k) // g.split_k >= 4                    # slices keep a useful number of K slabs
+                assert lib.tnx_gemm_workspace_bytes(ctypes.byref(g)) == 65536 + g.split_k * cut * g.block_m * g.block_n * 4
+            else:
+                assert g.tail_tiles == 0 and lib.tnx_gemm_workspace_bytes(ctypes.byref(g)) == 0
+
+
+def test_default_config_of_the_benchmark_shapes():
+    lib = _C.load()
+
+    def pick(dt, out, m, n, k):
+        g = args(m=m, n=n, k=k, stride_am=k, stride_bk=n, stride_cm=n, in_dtype=dt, out_dtype=out)
+        lib.tnx_gemm_default_config(ctypes.byref(g))
+        return (g.block_m, g.block_n, g.block_k, g.num_warps, g.num_stages, g.split_k, g.tail_tiles)
+
+    assert pick(_C.BF16, _C.BF16, 8192, 8192, 8192) == (256, 256, 64, 4, 2, 1, 0)
+    assert pick(_C.BF16, _C.BF16, 4096, 28672, 4096) == (256, 256, 64, 4, 2, 1, 0)
+    assert pick(_C.I8, _C.I32, 8192, 8192, 8192) == (256, 256, 128, 4, 2, 1, 0)
+    assert pick(_C.F16, _C.F16, 1024, 768, 512) == (64, 64, 64, 4, 4, 1, 0)
+    assert pick(_C.BF16, _C.BF16, 16, 4096, 14336) == (64, 128, 64, 8, 3, 8, 0)
+    # 576 tiles of 256x256 are 2.25 waves of 256 CUs: the last 64 tiles are cut four ways
+    assert pick(_C.BF16, _C.BF16, 6144, 6144, 6144) == (256, 256, 64, 4, 2, 4, 64)
+    # 400 tiles: 144 trailing tiles cannot be cut without spilling into another wave
+    assert pick(_C.BF16, _C.BF16, 5120, 5120, 8192) == (256, 256, 64, 4, 2, 1, 0)

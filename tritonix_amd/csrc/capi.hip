@@ -188,6 +188,7 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   const int64_t cus = 256;
   a->group_m = 8;
   a->split_k = 1;
+  a->tail_tiles = 0;
   a->block_k = bk;
   bool dma_ok;
   {
@@ -214,30 +215,42 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     a->block_m = a->m <= 64 ? 64 : 128; a->block_n = 128; a->num_stages = 2; a->num_warps = 4;
     return TNX_OK;
   }
-  // Pick the (tile, K split) pair with the smallest modelled time: waves of workgroups over 256 CUs,
-  // each tile costing its multiply-adds over the rate a CU sustains with that tile (relative rates
-  // measured on 8192^3: 256x256 1.0, 256x128 0.9, 128x128 0.7), plus a fixed cost for the split-K
-  // hand-over (partials through memory, one more round trip).  K is only cut when the tiles
-  // alone leave CUs idle, and never into pieces shorter than eight K slabs.
+  // Pick the tile and the K cut with the smallest modelled time.  A wave is 256 workgroups (one per CU); a tile
+  // costs its multiply-adds over the rate a CU sustains with that tile (relative rates measured on 8192^3 and
+  // 2048^2 x 8192: 256x256 1.0, 256x128 0.9, 128x128 0.75); a last, partial wave costs 0.75 of a full one (the
+  // part is power-limited: fewer busy CUs clock higher; measured 0.70-0.80 on 6144^3, 5120^2 x 8192,
+  // 4096 x 5120 x 4096).  Cutting K costs a hand-over: a fixed 9 us plus the slices the finishing workgroup
+  // reads back at about 60 GB/s.  Three shapes of launch are priced per tile: uncut; every tile cut (only when
+  // the tiles alone leave CUs idle); only the tiles of the partial wave cut (tail_tiles).  Slices never get
+  // shorter than eight K slabs.
   static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
-  static const double rate[] = {1.0, 0.9, 0.7, 0.5, 0.35};
+  static const double rate[] = {1.0, 0.9, 0.75, 0.5, 0.35};
   const int ncand = es == 1 ? 4 : 5;   // int8 rows of a 64-wide B tile are too short for the transposing read
   const double cu_flops = 5.5e12 * (es == 1 ? 1.7 : 1.0);          // per CU with the largest tile
+  const double launch = 3e-6, handover = 9e-6, readback = 60e9;
   const int64_t kt = (a->k + bk - 1) / bk;
   double best = 1e300;
-  int bi = 0, bs = 1;
+  int bi = ncand - 1, bs = 1, btail = 0;
+  auto offer = [&](double t, int i, int s, int tail) {
+    if (t < best * 0.97) { best = t; bi = i; bs = s; btail = tail; }   // ties go to the earlier (larger, less cut) choice
+  };
   for (int i = 0; i < ncand; ++i) {
     const int64_t tiles = ((a->m + cand[i][0] - 1) / cand[i][0]) * ((a->n + cand[i][1] - 1) / cand[i][1]);
-    for (int s = 1; s <= 16; s *= 2) {
-      if (s > 1 && (tiles * s > cus + cus / 4 || kt / s < 8)) break;
-      const int64_t waves = (tiles * s + cus - 1) / cus;
-      const double t = (double)waves * (2.0 * cand[i][0] * cand[i][1] * (double)a->k / s) / (cu_flops * rate[i]) +
-                       (s > 1 ? 4e-6 : 0.0) + 3e-6;
-      if (t < best * 0.97) { best = t; bi = i; bs = s; }             // ties go to the earlier (larger, unsplit) choice
+    const double tile_t = 2.0 * cand[i][0] * cand[i][1] * (double)a->k / (cu_flops * rate[i]);
+    const double slice_bytes = (double)cand[i][0] * cand[i][1] * 4;
+    const int64_t full = tiles / cus, rem = tiles % cus;
+    offer((double)full * tile_t + (rem ? 0.75 * tile_t : 0.0) + launch, i, 1, 0);
+    for (int s = 2; s <= 16; s *= 2) {
+      if (kt / s < 8) break;
+      if (full == 0 && tiles * s <= cus)                             // every tile cut (one wave at most)
+        offer(tile_t / s + handover + s * slice_bytes / readback + launch, i, s, 0);
+      if (full > 0 && rem > 0 && rem * s <= cus)                     // only the partial wave cut
+        offer((double)full * tile_t + tile_t / s + handover + s * slice_bytes / readback + launch, i, s, (int)rem);
     }
   }
   a->block_m = cand[bi][0]; a->block_n = cand[bi][1]; a->num_stages = cand[bi][2]; a->num_warps = cand[bi][3];
   a->split_k = bs;
+  a->tail_tiles = btail;
   return TNX_OK;
 }
 

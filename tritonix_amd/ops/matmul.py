@@ -206,6 +206,11 @@ def default_config(a, b, split=False):
            "num_stages": g.num_stages, "num_warps": g.num_warps}
     if split:
         cfg["split_k"] = max(2, g.split_k)
+    elif g.split_k > 1:
+        # shapes whose tiles alone leave CUs idle: the engine proposes a K cut for the plain kernel too
+        cfg["split_k"] = g.split_k
+    if g.tail_tiles > 0:
+        cfg["tail_tiles"] = g.tail_tiles
     return cfg
 
 
