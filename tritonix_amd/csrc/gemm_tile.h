@@ -40,7 +40,7 @@ struct GemmParams {
   const uint8_t* a;
   const uint8_t* b;
   uint8_t* c;
-  uint8_t* ws;            // split-K workspace: tile counters, then partials [split][m][n] (fp32 / int32)
+  uint8_t* ws;            // split-K workspace: tile counters, then the slices [slice][cut tile][wave][group][lane]
   int64_t m, n, k;
   int64_t sam, sak;       // element strides of A
   int64_t sbk, sbn;       // element strides of B
