@@ -37,7 +37,7 @@ enum tnx_dtype {
   TNX_BF16 = 1, /* bfloat16 */
   TNX_I8 = 2,   /* signed 8-bit */
   TNX_I32 = 3,  /* signed 32-bit (output of the int8 path) */
-  TNX_F32 = 4   /* binary32 (output only) */
+  TNX_F32 = 4   /* binary32: the type of split-K slices in the workspace; no entry point takes or returns it */
 };
 
 /* epilogues fused after the K loop (tritonix/ops/swiglu.py:98-104).
