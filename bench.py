@@ -121,6 +121,10 @@ def main():
     mm = importlib.import_module("tritonix_amd.ops.matmul")
     sg = importlib.import_module("tritonix_amd.ops.swiglu")
 
+    if not os.path.exists(_C.LIB_PATH):            # nothing built yet: build it; there is nothing to fall back to
+        from tritonix_amd import build as hip_build
+
+        hip_build.build(verbose=False)
     _C.load()
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)

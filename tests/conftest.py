@@ -17,6 +17,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the library that is built; only when there is none do they build it (hipcc, a few minutes)."""
+    from tritonix_amd import _C
+
+    if not os.path.exists(_C.LIB_PATH):
+        from tritonix_amd import build as hip_build
+
+        hip_build.build(verbose=False)
+
+
 @pytest.fixture(scope="session")
 def traces():
     with open(os.path.join(ROOT, "tests", "golden", "hand_traces.json")) as f:
