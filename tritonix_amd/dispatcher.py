@@ -1,199 +1,239 @@
-"""Per-shape backend dispatch: time every registered implementation once, keep the fastest.
+"""Per-signature choice between interchangeable implementations of one operation.
 
-API and behaviour follow tritonix/dispatcher.py of the reference:
-``_tuning_key`` (:18-30), ``_disk_key`` (:33-35), ``DynamicDispatcher``
-(:38-145) and ``dynamic_dispatch`` (:148-175).  The on-disk record keeps the
-reference's JSON schema ``{"op", "key", "winner", "timings"}`` and file name,
-but lives under ``$TRITONIX_CACHE_DIR`` (default ``~/.cache/tritonix_amd``)
-instead of Triton's cache directory, and the timer is the HIP-event
-``do_bench`` of this package (or any callable passed as ``bench_fn``).
+The first call with a new argument signature times every registered backend
+and remembers the winner; later calls go straight to it.  Public surface and
+observable behaviour are those of the reference's dispatcher
+(tritonix/dispatcher.py:18-35 for the two key functions, :38-145 for the
+class, :148-175 for the factory): ``register``, ``force_backend``,
+``clear_cache``, ``best_config``, the ``cache`` / ``timings`` dictionaries and
+the JSON record ``{"op", "key", "winner", "timings"}`` in a file called
+``backend_dispatch.json``.  Differences: records live under
+``$TRITONIX_CACHE_DIR`` (default ``~/.cache/tritonix_amd``) rather than in
+Triton's cache, the timer is this package's HIP-event ``do_bench`` unless a
+``bench_fn`` is injected, and ``alias`` lets one backend answer to two names.
 """
 from __future__ import annotations
 
+import contextlib
 import hashlib
 import inspect
 import json
 import logging
 import os
 import tempfile
-from contextlib import contextmanager
-from typing import Callable, Dict, List, Optional
-
-log = logging.getLogger(__name__)
+from typing import Any, Callable, Dict, Iterable, List, NamedTuple, Optional, Tuple
 
 __all__ = ["DynamicDispatcher", "dynamic_dispatch", "cache_dir"]
 
+_log = logging.getLogger(__name__)
+
 
 def cache_dir() -> str:
-    return os.environ.get("TRITONIX_CACHE_DIR") or os.path.join(os.path.expanduser("~"), ".cache", "tritonix_amd")
+    """Root of everything this package persists (dispatch records, tuned tile configs)."""
+    override = os.environ.get("TRITONIX_CACHE_DIR")
+    return override if override else os.path.join(os.path.expanduser("~"), ".cache", "tritonix_amd")
 
 
-def _is_tensor(v) -> bool:
-    return hasattr(v, "shape") and hasattr(v, "dtype") and hasattr(v, "stride")
+# ---------------------------------------------------------------------------
+# signatures
+# ---------------------------------------------------------------------------
+def _tensor_like(obj: Any) -> bool:
+    return all(hasattr(obj, attr) for attr in ("shape", "dtype", "stride"))
 
 
-def _describe(v) -> list:
-    return list(v.shape) + [str(v.dtype)]
+def _footprint(obj: Any) -> Tuple:
+    """What a tensor contributes to a signature: its extents, then its dtype as text."""
+    return (*obj.shape, str(obj.dtype))
 
 
 def _tuning_key(key_names: List[str], args: tuple, kwargs: dict, arg_names: List[str]) -> tuple:
-    """Shapes and dtypes of the keyed tensors, values of keyed scalars, then every other tensor argument."""
-    bound = dict(zip(arg_names, args))
-    bound.update(kwargs)
-    parts: list = []
+    """Signature of a call.
+
+    First the keyed arguments in the order the key lists them (a tensor gives
+    its footprint, anything else its value; names the call does not bind are
+    passed over), then the footprint of every remaining tensor argument in
+    binding order: positionals by parameter name, keywords after them.
+    """
+    call: Dict[str, Any] = {name: value for name, value in zip(arg_names, args)}
+    call.update(kwargs)
+    sig: List[Any] = []
     for name in key_names:
-        if name in bound:
-            v = bound[name]
-            parts.extend(_describe(v) if _is_tensor(v) else [v])
-    keyed = set(key_names)
-    for name, v in bound.items():
-        if name not in keyed and _is_tensor(v):
-            parts.extend(_describe(v))
-    return tuple(parts)
+        if name not in call:
+            continue
+        value = call[name]
+        sig += _footprint(value) if _tensor_like(value) else (value,)
+    for name, value in call.items():
+        if name not in key_names and _tensor_like(value):
+            sig += _footprint(value)
+    return tuple(sig)
 
 
-def _disk_key(op_name: str, backends: List[str], tuning_key: tuple) -> str:
-    text = "-".join([op_name, str(sorted(backends)), str(tuning_key)])
-    return hashlib.sha256(text.encode()).hexdigest()
+def _disk_key(op_name: str, backends: Iterable[str], tuning_key: tuple) -> str:
+    """Directory name of a record: sha256 over operation, sorted backend names and signature."""
+    material = f"{op_name}-{sorted(backends)}-{tuning_key}"
+    return hashlib.sha256(material.encode()).hexdigest()
 
 
+# ---------------------------------------------------------------------------
+# records on disk
+# ---------------------------------------------------------------------------
+class _Verdict(NamedTuple):
+    winner: str
+    timings: Dict[str, float]
+
+
+class _RecordStore:
+    """One small JSON file per (operation, backend set, signature); unreadable records count as absent."""
+
+    FILE_NAME = "backend_dispatch.json"
+
+    def __init__(self, op_name: str):
+        self.op_name = op_name
+
+    def _file(self, backends: Iterable[str], signature: tuple) -> str:
+        return os.path.join(cache_dir(), _disk_key(self.op_name, backends, signature), self.FILE_NAME)
+
+    def get(self, backends: Iterable[str], signature: tuple) -> Optional[_Verdict]:
+        try:
+            with open(self._file(backends, signature)) as fh:
+                raw = json.load(fh)
+            return _Verdict(raw["winner"], raw["timings"])
+        except FileNotFoundError:
+            return None
+        except (OSError, ValueError, KeyError, TypeError) as err:
+            _log.debug("[%s] unusable dispatch record: %s", self.op_name, err)
+            return None
+
+    def put(self, backends: Iterable[str], signature: tuple, verdict: _Verdict) -> None:
+        target = self._file(backends, signature)
+        body = {"op": self.op_name, "key": list(signature), "winner": verdict.winner, "timings": verdict.timings}
+        try:
+            os.makedirs(os.path.dirname(target), exist_ok=True)
+            handle, scratch = tempfile.mkstemp(dir=os.path.dirname(target), suffix=".tmp")
+            with os.fdopen(handle, "w") as fh:
+                json.dump(body, fh)
+            os.replace(scratch, target)          # readers never see a half-written record
+        except OSError as err:
+            _log.warning("[%s] dispatch record not written: %s", self.op_name, err)
+
+
+# ---------------------------------------------------------------------------
+# the dispatcher
+# ---------------------------------------------------------------------------
 class DynamicDispatcher:
-    """Callable that routes to the fastest registered backend for each argument signature."""
+    """Callable that sends each call to the backend that was fastest for its signature.
 
-    _CACHE_FILE = "backend_dispatch.json"
+    ``cache`` maps signature -> backend name, ``timings`` maps signature ->
+    ``{backend: ms}``; both are plain dictionaries a caller may inspect.  One
+    ``force_backend`` can be active at a time; the object is not thread-safe.
+    """
 
     def __init__(self, fn: Callable, key: List[str], arg_names: List[str], warmup: int = 25, rep: int = 100,
                  use_disk_cache: bool = True, bench_fn: Optional[Callable] = None):
-        self._fn = fn
-        self._key_names = key
-        self._arg_names = arg_names
-        self._warmup = warmup
-        self._rep = rep
-        self._disk = use_disk_cache
-        self._bench_fn = bench_fn
-        self._backends: Dict[str, Callable] = {}
-        self._forced: Optional[str] = None
-        self._aliases: Dict[str, str] = {}
-        self.cache: Dict[tuple, str] = {}
-        self.timings: Dict[tuple, Dict[str, float]] = {}
         self.__name__ = fn.__name__
         self.__doc__ = fn.__doc__
+        self._fn = fn
+        self._key_names, self._arg_names = key, arg_names
+        self._budget = {"warmup": warmup, "rep": rep}
+        self._bench_fn = bench_fn
+        self._store = _RecordStore(self.__name__) if use_disk_cache else None
+        self._backends: Dict[str, Callable] = {}
+        self._aliases: Dict[str, str] = {}
+        self._forced: Optional[str] = None
+        self.cache: Dict[tuple, str] = {}
+        self.timings: Dict[tuple, Dict[str, float]] = {}
 
+    # -- registration -------------------------------------------------------
     def register(self, name: str, impl: Callable) -> "DynamicDispatcher":
         self._backends[name] = impl
         return self
 
     def alias(self, alias: str, name: str) -> "DynamicDispatcher":
-        """Let ``force_backend(alias)`` select backend ``name`` (no second timing entry is created)."""
-        if name not in self._backends:
-            raise KeyError(f"Backend '{name}' not registered in '{self.__name__}'.")
-        self._aliases[alias] = name
+        """Make ``force_backend(alias)`` select backend ``name``; timings and records keep the one real name."""
+        self._aliases[alias] = self._resolve(name)
         return self
 
+    def _resolve(self, name: str) -> str:
+        real = self._aliases.get(name, name)
+        if real not in self._backends:
+            raise KeyError(f"Backend '{name}' not registered in '{self.__name__}'.")
+        return real
+
+    # -- calling ------------------------------------------------------------
     def __call__(self, *args, **kwargs):
         if not self._backends:
             raise RuntimeError(f"[{self.__name__}] No backends registered.")
         if self._forced is not None:
-            return self._backends[self._forced](*args, **kwargs)
-        key = _tuning_key(self._key_names, args, kwargs, self._arg_names)
-        if key not in self.cache:
-            self._bench_and_cache(key, args, kwargs)
-        return self._backends[self.cache[key]](*args, **kwargs)
+            chosen = self._forced
+        else:
+            signature = _tuning_key(self._key_names, args, kwargs, self._arg_names)
+            chosen = self.cache.get(signature)
+            if chosen is None:
+                chosen = self._decide(signature, args, kwargs)
+        return self._backends[chosen](*args, **kwargs)
 
-    # ------------------------------------------------------------------
-    def _timer(self) -> Callable:
-        if self._bench_fn is not None:
-            return self._bench_fn
-        from tritonix_amd.testing import do_bench
+    def _decide(self, signature: tuple, args: tuple, kwargs: dict) -> str:
+        """Winner for a signature seen for the first time in this process: a record on disk, else a race."""
+        names = list(self._backends)
+        verdict = self._store.get(names, signature) if self._store else None
+        if verdict is None or verdict.winner not in self._backends:
+            verdict = self._race(args, kwargs)
+            if self._store:
+                self._store.put(names, signature, verdict)
+        self.cache[signature], self.timings[signature] = verdict.winner, verdict.timings
+        return verdict.winner
 
-        return do_bench
-
-    def _bench_and_cache(self, key: tuple, args: tuple, kwargs: dict) -> None:
-        if self._disk and self._load_from_disk(key) is not None:
-            return
-        timer = self._timer()
-        results: Dict[str, float] = {}
+    def _race(self, args: tuple, kwargs: dict) -> _Verdict:
+        """Time every backend on this very call; one that raises simply does not finish."""
+        clock = self._bench_fn
+        if clock is None:
+            from tritonix_amd.testing import do_bench as clock
+        finished: Dict[str, float] = {}
         for name, impl in self._backends.items():
             try:
-                results[name] = timer(lambda: impl(*args, **kwargs), warmup=self._warmup, rep=self._rep)
-            except Exception as exc:  # a failing backend only loses the race
-                log.debug("[%s] backend '%s' skipped: %s", self.__name__, name, exc)
-        if not results:
+                finished[name] = clock(lambda: impl(*args, **kwargs), **self._budget)
+            except Exception as err:
+                _log.debug("[%s] backend '%s' dropped out: %s", self.__name__, name, err)
+        if not finished:
             raise RuntimeError(f"[{self.__name__}] All backends failed.")
-        winner = min(results, key=results.get)
-        log.info("[%s] %s", self.__name__, "  ".join(f"{n}={v:.3f}ms" for n, v in results.items()))
-        self.cache[key] = winner
-        self.timings[key] = results
-        if self._disk:
-            self._save_to_disk(key, results, winner)
+        _log.info("[%s] %s", self.__name__, ", ".join(f"{n}: {ms:.3f} ms" for n, ms in finished.items()))
+        return _Verdict(min(finished, key=finished.__getitem__), finished)
 
-    def _disk_path(self, key: tuple) -> str:
-        return os.path.join(cache_dir(), _disk_key(self.__name__, list(self._backends.keys()), key), self._CACHE_FILE)
-
-    def _load_from_disk(self, key: tuple) -> Optional[str]:
-        try:
-            path = self._disk_path(key)
-            if not os.path.exists(path):
-                return None
-            with open(path) as f:
-                data = json.load(f)
-            if data["winner"] not in self._backends:
-                return None
-            self.cache[key] = data["winner"]
-            self.timings[key] = data["timings"]
-            return data["winner"]
-        except Exception as exc:
-            log.debug("[%s] disk miss: %s", self.__name__, exc)
-            return None
-
-    def _save_to_disk(self, key: tuple, results: Dict[str, float], winner: str) -> None:
-        try:
-            path = self._disk_path(key)
-            os.makedirs(os.path.dirname(path), exist_ok=True)
-            payload = json.dumps({"op": self.__name__, "key": list(key), "winner": winner, "timings": results})
-            fd, tmp = tempfile.mkstemp(dir=os.path.dirname(path), suffix=".tmp")
-            with os.fdopen(fd, "w") as f:
-                f.write(payload)
-            os.replace(tmp, path)
-        except Exception as exc:
-            log.warning("[%s] disk write failed: %s", self.__name__, exc)
-
-    # ------------------------------------------------------------------
-    @contextmanager
+    # -- control ------------------------------------------------------------
+    @contextlib.contextmanager
     def force_backend(self, name: str):
-        name = self._aliases.get(name, name)
-        if name not in self._backends:
-            raise KeyError(f"Backend '{name}' not registered in '{self.__name__}'.")
-        self._forced = name
+        """Inside the block every call goes to ``name`` (or what it aliases); nothing is timed or remembered."""
+        self._forced = self._resolve(name)
         try:
             yield
         finally:
             self._forced = None
 
     def clear_cache(self) -> None:
-        """Forget the in-memory winners and timings (records on disk stay)."""
+        """Forget winners and timings held in memory; records on disk stay and are found again."""
         self.cache.clear()
         self.timings.clear()
 
     def best_config(self) -> Dict[tuple, str]:
+        """A copy of signature -> winning backend."""
         return dict(self.cache)
 
 
 def dynamic_dispatch(backends: Optional[Dict[str, Callable]] = None, key: Optional[List[str]] = None, warmup: int = 25,
                      rep: int = 100, use_disk_cache: bool = True, bench_fn: Optional[Callable] = None):
-    """Build a dispatcher from a ``{name: impl}`` dict, or use as ``@dynamic_dispatch(key=[...])``.
+    """``dynamic_dispatch({"name": impl, ...}, key=[...])`` returns a dispatcher named after the first
+    implementation (its docstring and parameter names too); ``@dynamic_dispatch(key=[...])`` on a stub returns an
+    empty dispatcher to ``register`` backends on."""
 
-    With a dict the dispatcher takes its name, docstring and argument names
-    from the first backend.
-    """
+    def wrap(template: Callable) -> DynamicDispatcher:
+        params = list(inspect.signature(template).parameters)
+        return DynamicDispatcher(template, key=list(key or []), arg_names=params, warmup=warmup, rep=rep,
+                                 use_disk_cache=use_disk_cache, bench_fn=bench_fn)
 
-    def make(fn: Callable) -> DynamicDispatcher:
-        return DynamicDispatcher(fn, key=key or [], arg_names=list(inspect.signature(fn).parameters.keys()),
-                                 warmup=warmup, rep=rep, use_disk_cache=use_disk_cache, bench_fn=bench_fn)
-
-    if backends is not None:
-        d = make(next(iter(backends.values())))
-        for name, impl in backends.items():
-            d.register(name, impl)
-        return d
-    return make
+    if backends is None:
+        return wrap
+    impls = list(backends.items())
+    dispatcher = wrap(impls[0][1])
+    for name, impl in impls:
+        dispatcher.register(name, impl)
+    return dispatcher

@@ -14,7 +14,7 @@ both names are bound to it here.
 from __future__ import annotations
 
 import random
-from typing import Callable, Dict, Iterator, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, Iterable, Iterator, List, Optional, Sequence, Tuple
 
 from tritonix_amd.utils.spaces import SpaceConfig
 
@@ -22,179 +22,168 @@ __all__ = ["MonotonicCascadeTrie", "CoordinateUnimodalFunction", "CoordinateMono
 
 
 def _dominates_config(failure: Sequence[int], candidate: Sequence[int]) -> bool:
-    """candidate is at least failure in every coordinate"""
-    return all(c >= f for c, f in zip(candidate, failure))
+    """True when ``candidate`` is no smaller than ``failure`` anywhere (so it fails too)."""
+    for c, f in zip(candidate, failure):
+        if c < f:
+            return False
+    return True
 
 
 def _dominates_dim(failure: int, candidate: int, rank: int = 0) -> bool:
-    return candidate >= failure
-
-
-class _Node:
-    __slots__ = ("kids", "terminal")
-
-    def __init__(self):
-        self.kids: Dict[int, "_Node"] = {}
-        self.terminal = False
+    """One-coordinate version of the order above; ``rank`` is the dimension, unused by the default order."""
+    return not candidate < failure
 
 
 def _centre_out(n: int) -> Iterator[int]:
-    """n//2, then alternately one step below and one step above, until 0..n-1 is used up."""
-    mid = n // 2
-    yield mid
-    below, above = mid - 1, mid + 1
-    while below >= 0 or above < n:
-        if below >= 0:
-            yield below
-            below -= 1
-        if above < n:
-            yield above
-            above += 1
+    """0..n-1 starting from n//2 and fanning out: one below, one above, two below, two above, ..."""
+    start = n // 2
+    yield start
+    for step in range(1, n):
+        if start - step >= 0:
+            yield start - step
+        if start + step < n:
+            yield start + step
 
 
 class MonotonicCascadeTrie:
-    """Prefix tree over the minimal failures of a monotone search space."""
+    """The minimal failures of a monotone search space, and what they leave alive.
+
+    Failures are kept as an antichain (no stored failure is >= another one),
+    grouped by their leading coordinate so that a query only looks at groups
+    whose leading coordinate is small enough.  The two comparison functions
+    can be replaced to order the space differently; the defaults are the
+    componentwise ">=".
+    """
 
     def __init__(self, space: SpaceConfig, config_comparison_func: Callable = _dominates_config,
                  dimension_comparison_func: Callable = _dominates_dim):
         self.shape = space.shape
         self.dimensions = len(self.shape)
-        self._minimal_failures: List[Tuple[int, ...]] = []
-        self._root = _Node()
         self._config_compare = config_comparison_func
         self._dim_compare = dimension_comparison_func
+        self._minimal_failures: List[Tuple[int, ...]] = []
+        self._by_lead: Dict[int, List[Tuple[int, ...]]] = {}
 
     # -- queries ---------------------------------------------------------
     def is_pruned(self, config_idx) -> bool:
-        """True when some recorded failure is <= config_idx in every coordinate."""
-        if len(config_idx) != self.dimensions:
+        """Does a recorded failure sit at or below ``config_idx`` in every coordinate?"""
+        cfg = tuple(config_idx)
+        if len(cfg) != self.dimensions:
             raise ValueError(f"is_pruned expects a full-length config of length {self.dimensions}")
-        return self._covered(tuple(config_idx), 0, self._root)
-
-    def _covered(self, cfg: Tuple[int, ...], depth: int, node: _Node) -> bool:
-        if node.terminal:
-            return True
-        if depth == len(cfg):
-            return False
-        here = cfg[depth]
-        for fail_idx, child in node.kids.items():
-            if self._dim_compare(fail_idx, here, depth) and self._covered(cfg, depth + 1, child):
-                return True
+        if not cfg:
+            return bool(self._minimal_failures)
+        for lead, group in self._by_lead.items():
+            if not self._dim_compare(lead, cfg[0], 0):
+                continue
+            for failure in group:
+                if all(self._dim_compare(f, c, d) for d, (f, c) in enumerate(zip(failure, cfg)) if d):
+                    return True
         return False
 
     def _is_prefix_doomed(self, prefix) -> bool:
-        """A prefix is dead when even its all-zero completion is pruned."""
-        prefix = tuple(prefix)
-        if not prefix:
+        """Nothing that starts with ``prefix`` survives: its smallest completion (zeros) is already pruned."""
+        lead = tuple(prefix)
+        if len(lead) == 0:
             return False
-        return self.is_pruned(prefix + (0,) * (self.dimensions - len(prefix)))
+        padding = (0,) * (self.dimensions - len(lead))
+        return self.is_pruned(lead + padding)
 
     # -- updates ---------------------------------------------------------
     def prune(self, failed_config) -> None:
-        """Record a failure; failures it makes redundant are dropped."""
+        """Add a failure unless a stored one already implies it; stored ones it implies are dropped."""
         if self.is_pruned(failed_config):
             return
-        kept = [f for f in self._minimal_failures if not self._config_compare(failed_config, f)]
-        kept.append(failed_config)
-        self._minimal_failures = kept
-        self._root = _Node()
-        for f in kept:
-            node = self._root
-            for idx in f:
-                node = node.kids.setdefault(idx, _Node())
-            node.terminal = True
+        survivors = [old for old in self._minimal_failures if not self._config_compare(failed_config, old)]
+        survivors.append(failed_config)
+        self._minimal_failures = survivors
+        self._by_lead = {}
+        for failure in survivors:
+            self._by_lead.setdefault(failure[0] if len(failure) else 0, []).append(tuple(failure))
 
     # -- enumeration -----------------------------------------------------
-    def _first_survivor(self, prefix: Tuple[int, ...], order: Callable[[int], Sequence[int]]) -> Optional[Tuple[int, ...]]:
-        if self._is_prefix_doomed(prefix):
-            return None
-        if len(prefix) == self.dimensions:
-            return prefix
-        for idx in order(self.shape[len(prefix)]):
-            found = self._first_survivor(prefix + (idx,), order)
-            if found is not None:
-                return found
-        return None
+    def _survivors(self, order: Callable[[int], Iterable[int]]) -> Iterator[Tuple[int, ...]]:
+        """Depth-first over index prefixes, children of a prefix in ``order``; dead prefixes are not entered.
+
+        Lazy: a ``prune()`` between two items changes what comes next, which the tuner relies on.
+        """
+        pending: List[Tuple[int, ...]] = [()]
+        while pending:
+            prefix = pending.pop()
+            if self._is_prefix_doomed(prefix):
+                continue
+            if len(prefix) == self.dimensions:
+                yield prefix
+                continue
+            children = [prefix + (i,) for i in order(self.shape[len(prefix)])]
+            pending.extend(reversed(children))
 
     def get_random_unpruned(self) -> Optional[Tuple[int, ...]]:
-        def shuffled(n):
-            idx = list(range(n))
-            random.shuffle(idx)
-            return idx
-
-        return self._first_survivor((), shuffled)
+        """Some survivor, dimensions explored in random order of their values; ``None`` if nothing survives."""
+        return next(self._survivors(lambda n: random.sample(range(n), n)), None)
 
     def get_mid_point_unpruned(self) -> Optional[Tuple[int, ...]]:
-        return self._first_survivor((), lambda n: list(_centre_out(n)))
-
-    def _walk(self, prefix: Tuple[int, ...], order: Callable[[int], Sequence[int]]) -> Iterator[Tuple[int, ...]]:
-        # lazy on purpose: a prune() issued by the consumer between two
-        # yields changes what is produced afterwards
-        if self._is_prefix_doomed(prefix):
-            return
-        if len(prefix) == self.dimensions:
-            yield prefix
-            return
-        for idx in order(self.shape[len(prefix)]):
-            yield from self._walk(prefix + (idx,), order)
+        """The first survivor of the centre-out walk; ``None`` if nothing survives."""
+        return next(self._survivors(_centre_out), None)
 
     def generate_all_unpruned(self) -> Iterator[Tuple[int, ...]]:
         """Surviving index tuples in lexicographic order."""
-        yield from self._walk((), range)
+        return self._survivors(range)
 
     def generate_all_unpruned_midpoint(self) -> Iterator[Tuple[int, ...]]:
         """Surviving index tuples, every dimension visited centre-out."""
-        yield from self._walk((), _centre_out)
+        return self._survivors(_centre_out)
+
+
+def _window(seen: Dict[int, float], size: int) -> Tuple[int, int]:
+    """Index range that can still hold the minimum of a unimodal sequence observed at ``seen``.
+
+    Walking away from the best observation, the nearest observation that is strictly worse closes the range on
+    that side (the minimum cannot lie beyond a point where the function has started to rise).
+    """
+    at = sorted(seen)
+    best = min(seen, key=seen.__getitem__)      # among equal values: the one observed first
+    floor = seen[best]
+    above = next((i for i in at if i > best and seen[i] > floor), None)
+    below = next((i for i in reversed(at) if i < best and seen[i] > floor), None)
+    return (0 if below is None else below + 1, size - 1 if above is None else above - 1)
 
 
 class CoordinateUnimodalFunction:
     """Coordinate-wise unimodality pruner.
 
-    Fix all coordinates but one: along the free one the function is assumed to
-    have a single minimum.  After two or more observations in such a slice,
-    the first observation right of the best one that is strictly worse caps
-    the window from above, the first one left of it that is strictly worse
-    caps it from below.  A config outside the window of any of its slices is
-    pruned.  Windows are recomputed from all observations at every record.
+    Fix all coordinates but one: along the free one the timing is assumed to have a single minimum.  Every
+    observation belongs to one such line per dimension; once a line holds two or more observations the range
+    that can still contain its minimum is recomputed from all of them (it may widen again when a new best turns
+    up).  A config is pruned when, along any dimension, it lies outside the range of its line.
     """
 
     def __init__(self, space: SpaceConfig):
         self.dim_sizes = list(space.shape)
         self.n_dims = len(self.dim_sizes)
-        self._obs: List[Dict[tuple, Dict[int, float]]] = [dict() for _ in range(self.n_dims)]
-        self._ranges: List[Dict[tuple, Tuple[int, int]]] = [dict() for _ in range(self.n_dims)]
+        # per dimension: line (the other coordinates) -> {index along the dimension: value} / -> (lo, hi)
+        self._obs: List[Dict[tuple, Dict[int, float]]] = [{} for _ in self.dim_sizes]
+        self._ranges: List[Dict[tuple, Tuple[int, int]]] = [{} for _ in self.dim_sizes]
 
     @staticmethod
     def _slice_key(idx: Tuple[int, ...], d: int) -> tuple:
         return idx[:d] + idx[d + 1:]
 
     def record(self, config_idx, value: float) -> None:
-        config_idx = tuple(config_idx)
-        for d in range(self.n_dims):
-            key = self._slice_key(config_idx, d)
-            seen = self._obs[d].setdefault(key, {})
-            seen[config_idx[d]] = value
-            if len(seen) < 2:
-                continue
-            best = min(seen, key=seen.__getitem__)
-            floor = seen[best]
-            lo, hi = 0, self.dim_sizes[d] - 1
-            for i in sorted(seen):
-                if i > best and seen[i] > floor:
-                    hi = i - 1
-                    break
-            for i in sorted(seen, reverse=True):
-                if i < best and seen[i] > floor:
-                    lo = i + 1
-                    break
-            if lo > 0 or hi < self.dim_sizes[d] - 1:
-                self._ranges[d][key] = (lo, hi)
+        point = tuple(config_idx)
+        for d, size in enumerate(self.dim_sizes):
+            line = self._slice_key(point, d)
+            seen = self._obs[d].setdefault(line, {})
+            seen[point[d]] = value
+            if len(seen) >= 2:
+                window = _window(seen, size)
+                if window != (0, size - 1):
+                    self._ranges[d][line] = window
 
     def is_pruned(self, config_idx) -> bool:
-        config_idx = tuple(config_idx)
+        point = tuple(config_idx)
         for d in range(self.n_dims):
-            window = self._ranges[d].get(self._slice_key(config_idx, d))
-            if window is not None and not (window[0] <= config_idx[d] <= window[1]):
+            window = self._ranges[d].get(self._slice_key(point, d))
+            if window is not None and not window[0] <= point[d] <= window[1]:
                 return True
         return False
 
