@@ -1,6 +1,15 @@
-from tritonix_amd.ops.matmul import (matmul, triton_matmul, hip_matmul, matmul_splitk, matmul_kernel,
-                                     gemm_splitk_kernel)
-from tritonix_amd.ops.swiglu import glu_kernel, glu, swiglu, swiglu_ffn, fused_glu
+"""Operators built on the HIP tile kernels: GEMM / split-K GEMM (``matmul``) and the gated GEMM (``swiglu``)."""
+import importlib
 
-__all__ = ["matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel", "gemm_splitk_kernel",
-           "glu_kernel", "glu", "swiglu", "swiglu_ffn", "fused_glu"]
+# ``ops.matmul`` names both a module and, once imported, the dispatcher it defines: bind the names explicitly
+_matmul_module = importlib.import_module("tritonix_amd.ops.matmul")
+_swiglu_module = importlib.import_module("tritonix_amd.ops.swiglu")
+
+__all__ = []
+for _module, _names in ((_matmul_module, ("matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel",
+                                           "gemm_splitk_kernel")),
+                        (_swiglu_module, ("glu_kernel", "glu", "swiglu", "swiglu_ffn", "fused_glu"))):
+    for _name in _names:
+        globals()[_name] = getattr(_module, _name)
+        __all__.append(_name)
+del _module, _names, _name
