@@ -140,3 +140,19 @@ def test_package_matmul_dispatcher_shape():
     assert torch.equal(out, torch.full((2, 4), 3.0))
     with matmul.force_backend("hip"):                  # alias of "triton"
         assert matmul._forced == "triton"
+
+
+def test_default_timer_is_the_package_do_bench(cache_dir, monkeypatch):
+    """Without ``bench_fn`` the race is timed by ``tritonix_amd.testing.do_bench`` with the dispatcher's budgets."""
+    import tritonix_amd.testing
+
+    seen = []
+
+    def stand_in(fn, warmup=25, rep=100):
+        seen.append((warmup, rep))
+        return {"fast": 1.0, "slow": 2.0}[fn()]
+
+    monkeypatch.setattr(tritonix_amd.testing, "do_bench", stand_in)
+    d = dynamic_dispatch({"s": slow, "f": fast}, key=["a", "b"], warmup=5, rep=11)
+    assert d(torch.empty(3, 3), torch.empty(3, 3)) == "fast"
+    assert seen == [(5, 11), (5, 11)]
