@@ -213,7 +213,7 @@ def main():
                "kind": "port", "sample": f"torch fp32 CPU matmul, first {rows_n} of {m} rows of A x full B, median of {reps}"}
 
     out = {
-        "metric": "TFLOP/s + % of dense MFMA peak, bf16 GEMM 8192^3 on 1xMI355X",
+        "metric": "TFLOP/s + % of dense MFMA peak, bf16 GEMM 8192\u00b3 on 1\u00d7MI355X",
         "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
