@@ -133,13 +133,39 @@ def test_package_matmul_dispatcher_shape():
     from tritonix_amd import matmul
 
     assert matmul.__name__ == "triton_matmul"
-    assert set(matmul._backends) == {"triton", "pytorch"}
+    assert set(matmul._backends) == {"triton", "splitk", "skinny", "pytorch"}
+    # the vendor library is reachable when forced, but is not a contender: the race is among HIP variants only
+    assert set(matmul._contenders()) == {"triton", "splitk", "skinny"}
     assert matmul._arg_names == ["a", "b"] and matmul._key_names == ["a", "b"]
     with matmul.force_backend("pytorch"):
         out = matmul(torch.ones(2, 3), torch.ones(3, 4))
     assert torch.equal(out, torch.full((2, 4), 3.0))
     with matmul.force_backend("hip"):                  # alias of "triton"
         assert matmul._forced == "triton"
+
+
+def test_unraced_backend_is_never_timed_and_never_wins(cache_dir):
+    t = Timer({"fast": 5.0, "slow": 9.0, "oracle": 0.1})
+    d = dynamic_dispatch({"s": slow, "f": fast}, key=["a", "b"], bench_fn=t)
+    assert d.register("ref", lambda a, b: "oracle", raced=False) is d
+    a, b = torch.empty(4, 2), torch.empty(2, 3)
+    assert d(a, b) == "fast"
+    assert [c[0] for c in t.calls] == ["slow", "fast"]              # "ref" was not timed
+    key = (4, 2, "torch.float32", 2, 3, "torch.float32")
+    assert d.cache == {key: "f"} and "ref" not in d.timings[key]
+    with d.force_backend("ref"):
+        assert d(a, b) == "oracle"
+    # a record on disk that names an un-raced backend as the winner (written when it was still raced) is ignored
+    d2 = dynamic_dispatch({"s": slow, "f": fast}, key=["a", "b"], bench_fn=Timer({"fast": 1.0, "slow": 2.0, "oracle": 0.1}))
+    d2.register("ref", lambda a, b: "oracle")
+    c, e = torch.empty(5, 2), torch.empty(2, 3)
+    assert d2(c, e) == "oracle"
+    d3 = dynamic_dispatch({"s": slow, "f": fast}, key=["a", "b"], bench_fn=Timer({"fast": 1.0, "slow": 2.0}))
+    d3.register("ref", lambda a, b: "oracle", raced=False)
+    assert d3(c, e) == "fast"
+    # registering again as raced puts it back into the race
+    d3.register("ref", lambda a, b: "oracle", raced=True)
+    assert "ref" in d3._contenders()
 
 
 def test_default_timer_is_the_package_do_bench(cache_dir, monkeypatch):

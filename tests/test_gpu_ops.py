@@ -32,7 +32,7 @@ def test_matmul_correctness(device, M, N, K):
     assert close(torch.matmul(a, b), out), f"max diff: {(torch.matmul(a, b) - out).abs().max()}"
     ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
     assert ok and rel <= 1e-2
-    assert (M, N, K, torch.float16) in mm._matmul_cfg
+    assert (M, N, K, torch.float16, True) in mm._matmul_cfg
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 512, 512), (2048, 2048, 2048)])
@@ -54,7 +54,7 @@ def test_dispatch_caches_winner(device):
     b = torch.randn(1024, 1024, device=device, dtype=torch.float16)
     out1 = matmul(a, b)
     assert len(matmul.cache) == 1
-    assert list(matmul.cache.values())[0] in ("triton", "pytorch")
+    assert list(matmul.cache.values())[0] in ("triton", "splitk", "skinny")
     assert list(matmul.cache)[0] == (1024, 1024, "torch.float16", 1024, 1024, "torch.float16")
     out2 = matmul(a, b)
     assert torch.allclose(out1.float(), out2.float(), atol=1.0, rtol=1e-2)
@@ -84,7 +84,7 @@ def test_matmul_splitk(device):
     out = tritonix_amd.matmul_splitk(a.to(device), b.to(device))
     ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
     assert ok and rel <= 1e-2
-    assert mm._splitk_cfg[(16, 2048, 7168, 4, torch.bfloat16)]["split_k"] >= 2
+    assert mm._splitk_cfg[(16, 2048, 7168, 4, torch.bfloat16, True)]["split_k"] >= 2
 
 
 def test_glu_and_swiglu_wrappers(device):
@@ -106,7 +106,7 @@ def test_glu_and_swiglu_wrappers(device):
 
 def test_int8_through_the_dispatcher(device):
     a, b = oracle.make_inputs("C5", scale_down=16)
-    out = tritonix_amd.matmul(a.to(device), b.to(device))       # torch has no int8 GPU matmul: "pytorch" drops out
+    out = tritonix_amd.matmul(a.to(device), b.to(device))
     assert out.dtype == torch.int32
     assert torch.equal(out.cpu(), oracle.reference_matmul(a, b))
 
@@ -189,8 +189,57 @@ def test_tuned_config_is_reused_from_disk(device, tmp_path, monkeypatch):
     b = torch.randn(256, 512, device=device, dtype=torch.float16)
     mm._matmul_cfg.clear()
     out1 = tritonix_amd.triton_matmul(a, b)
-    picked = mm._matmul_cfg[(384, 512, 256, torch.float16)]
-    assert mm.load_tuned("matmul", (384, 512, 256, torch.float16)) == picked
+    picked = mm._matmul_cfg[(384, 512, 256, torch.float16, True)]
+    assert mm.load_tuned("matmul", (384, 512, 256, torch.float16, True)) == picked
     mm._matmul_cfg.clear()
     monkeypatch.setattr(mm.matmul_kernel, "tune", lambda *a, **k: pytest.fail("tuned again despite the disk record"))
     assert torch.equal(tritonix_amd.triton_matmul(a, b), out1)
+
+
+def test_memoised_config_follows_the_operand_layout(device, monkeypatch):
+    """A tile remembered for row-major operands must not be handed to a transposed view of the same shape
+    (most tiles exist with the direct-to-LDS loader only), and the other way round."""
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    mm._matmul_cfg.clear()
+    g = torch.Generator("cpu").manual_seed(9)
+    a = torch.randn(512, 256, generator=g).half()
+    w = torch.randn(384, 256, generator=g).half()            # w.t() is [256, 384] with stride_bn != 1
+    ref = oracle.reference_matmul(a, w.t())
+    ad, wd = a.to(device), w.to(device)
+    b_contig = wd.t().contiguous()
+    out1 = tritonix_amd.triton_matmul(ad, b_contig)
+    out2 = tritonix_amd.triton_matmul(ad, wd.t())
+    out3 = tritonix_amd.triton_matmul(ad, b_contig)
+    for out in (out1, out2, out3):
+        assert oracle.within_tolerance(out, ref)[0]
+    assert torch.equal(out1, out3)
+    assert mm._matmul_cfg[(512, 384, 256, torch.float16, True)] != mm._matmul_cfg[(512, 384, 256, torch.float16, False)]
+    # a misaligned base pointer is the second layout class too
+    flat = torch.zeros(512 * 256 + 8, dtype=torch.float16, device=device)
+    a_off = flat[1:1 + 512 * 256].view(512, 256)
+    a_off.copy_(ad)
+    assert not mm.dma_layout(a_off, b_contig)
+    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_off, b_contig), ref)[0]
+    # a memo entry the engine refuses for these operands is replaced, not raised
+    mm._matmul_cfg[(512, 384, 256, torch.float16, False)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, True)],
+                                                                 block_m=256, block_n=256, num_stages=2, num_warps=4)
+    assert oracle.within_tolerance(tritonix_amd.triton_matmul(ad, wd.t()), ref)[0]
+    mm._matmul_cfg.clear()
+
+
+@pytest.mark.parametrize("name,scale", [("C1", 1), ("C2", 4), ("C3", 2), ("C5", 8)])
+def test_unforced_dispatch_never_selects_the_vendor_library(device, name, scale, tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITONIX_CACHE_DIR", str(tmp_path))
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    matmul = tritonix_amd.matmul
+    matmul.clear_cache()
+    a, b = oracle.make_inputs(name, scale_down=scale)
+    out = matmul(a.to(device), b.to(device))
+    (key, winner), = matmul.cache.items()
+    assert winner in ("triton", "splitk", "skinny") and "pytorch" not in matmul.timings[key]
+    ref = oracle.reference_matmul(a, b)
+    if a.dtype == torch.int8:
+        assert torch.equal(out.cpu(), ref)
+    else:
+        assert oracle.within_tolerance(out, ref)[0]
+    matmul.clear_cache()

@@ -40,6 +40,22 @@ def check_fp(out, ref):
     assert rel <= REL
 
 
+def whole_matrix_identity(out, a64, b64, rel_bound=2e-3):
+    """A check that touches every element of a result too large for an element-wise CPU comparison:
+    row sums  C.1 == A.(B.1)  and column sums  1.C == (1.A).B , right-hand sides in float64 on the CPU.
+    The left-hand sides differ from them only by the 16-bit rounding of each output element, whose sum over a
+    row has a standard deviation of about 2^-9 * rms(C) * sqrt(n): the bound is set at many times that,
+    while a tile left unwritten or written to the wrong place moves a sum by the size of the tile's content."""
+    c = out.double().cpu()
+    n_cols = c.shape[1]
+    want_rows = a64 @ b64.sum(dim=1)
+    want_cols = a64.sum(dim=0) @ b64
+    scale = float(c.abs().mean()) * n_cols ** 0.5          # size of a row sum of independent entries
+    assert float((c.sum(dim=1) - want_rows).abs().max()) <= rel_bound * scale * 8
+    scale_c = float(c.abs().mean()) * c.shape[0] ** 0.5
+    assert float((c.sum(dim=0) - want_cols).abs().max()) <= rel_bound * scale_c * 8
+
+
 F16_TILES = [cfg(128, 128, 64, 4, 2), cfg(128, 128, 64, 4, 3), cfg(256, 256, 64, 4, 2), cfg(64, 128, 64, 4, 3, gm=4),
              cfg(128, 128, 64, 8, 2), cfg(256, 256, 64, 8, 2), cfg(64, 128, 64, 8, 3)]
 
@@ -66,8 +82,10 @@ def test_c2_bf16_full_size_rows_and_linearity(device):
     ad, bd = a.to(device), b.to(device)
     config = cfg(256, 256, 64, 4, 2)
     out = gemm(ad, bd, config)
-    rows = torch.tensor([0, 1, 255, 256, 4095, 4096, 8190, 8191] + list(range(1000, 8000, 500)))
+    # one row out of every 256-row tile (at a different offset inside each) plus the edges of the matrix
+    rows = torch.tensor(sorted({0, 1, 255, 256, 4095, 4096, 8190, 8191} | {256 * t + (37 * t + 5) % 256 for t in range(32)}))
     check_fp(out[rows.to(device)], oracle.reference_matmul(a[rows], b))
+    whole_matrix_identity(out, a.double(), b.double())
     # scaling an operand by a power of two scales every product and partial sum exactly
     out2 = gemm(ad * 2, bd, config)
     assert torch.equal(out2, out * 2)
@@ -116,11 +134,21 @@ def test_c4_glu_scaled(device, activation, config):
 def test_c4_glu_full_size_rows(device):
     x, w12 = oracle.make_inputs("C4")
     xd, wd = x.to(device), w12.to(device)
-    rows = torch.tensor([0, 255, 256, 2047, 2048, 4095] + list(range(100, 4000, 390)))
+    rows = torch.tensor(sorted({0, 255, 256, 2047, 2048, 4095} | {256 * t + (53 * t + 11) % 256 for t in range(16)}))
     for act in ("silu", "sigmoid"):
         z = torch.empty((4096, 14336), device=device, dtype=torch.bfloat16)
         run(glu_kernel, xd, wd, z, cfg(256, 256, 64, 4, 2), activation=act)
         check_fp(z[rows.to(device)], oracle.reference_glu(x[rows], w12, act))
+    # every element of a whole result: the un-activated gate makes Z = (x W1) * (x W2) elementwise, and the plain
+    # GEMM of the same operands through the same tile gives both factors; the products must agree within the two
+    # roundings, everywhere (the plain kernel is itself checked over the whole matrix by the test below)
+    z = torch.empty((4096, 14336), device=device, dtype=torch.bfloat16)
+    run(glu_kernel, xd, wd, z, cfg(256, 256, 64, 4, 2), activation="identity")
+    y = gemm(xd, wd, cfg(256, 256, 64, 4, 2))
+    prod = y[:, 0::2].float() * y[:, 1::2].float()
+    err = (z.float() - prod).abs()
+    assert bool((err <= 2e-2 * prod.abs() + 1e-2 * prod.pow(2).mean().sqrt()).all())
+    whole_matrix_identity(y, x.double(), w12.double())
 
 
 # ---- C5: int8 -> int32, bit-exact -----------------------------------------------------

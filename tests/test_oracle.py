@@ -172,6 +172,29 @@ def test_glu_closed_forms_and_interleave_convention():
 
 
 # ---- seeded inputs -------------------------------------------------------------------
+def test_reference_matmul_float_branch_against_float64():
+    """The fp32 CPU matmul the parity bar is anchored on, against a float64 numpy product of the same 16-bit
+    inputs: fp32 accumulation over K=4096 terms of size ~1 stays within a few 1e-6 of the exact product relative
+    to sqrt(K), far inside the 1e-2 bar; a transposed operand, a dropped K tail or a wrong upcast would not."""
+    g = torch.Generator("cpu").manual_seed(21)
+    for dt in (torch.float16, torch.bfloat16):
+        a = torch.randn(96, 4096, generator=g).to(dt)
+        b = torch.randn(4096, 80, generator=g).to(dt)
+        want = a.double().numpy() @ b.double().numpy()
+        got = oracle.reference_matmul(a, b)
+        assert got.dtype == torch.float32 and got.shape == (96, 80)
+        assert np.abs(got.double().numpy() - want).max() <= 2e-5 * np.sqrt(4096.0)
+        # non-contiguous views must be honoured as views, not reinterpreted
+        at = a.t().contiguous().t()
+        assert torch.equal(oracle.reference_matmul(at, b), got)
+    # within_tolerance itself: exact passes, an error of 3 % of the rms on one element fails
+    ref = torch.randn(8, 8, generator=g)
+    assert oracle.within_tolerance(ref.clone(), ref)[0]
+    bad = ref.clone()
+    bad[3, 4] += 0.03 * float(ref.pow(2).mean().sqrt()) + 0.02 * float(ref[3, 4].abs())
+    assert not oracle.within_tolerance(bad, ref)[0]
+
+
 def test_seeded_inputs_are_reproducible_and_shaped():
     a1, b1 = oracle.make_inputs("C1")
     a2, b2 = oracle.make_inputs("C1")

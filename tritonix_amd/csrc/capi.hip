@@ -39,7 +39,15 @@ static int64_t lds_bytes_of(const tnx_gemm_args* a) {
   if (a->block_m <= 0 || a->block_n <= 0 || a->block_k <= 0 || a->num_stages <= 0) return -1;
   if (is_skinny_cfg(a)) return (int64_t)a->num_stages * SKINNY_NW * SKINNY_STEP_BYTES;
   int es = elem_size(a->in_dtype);
-  return (int64_t)a->num_stages * ((int64_t)a->block_m * a->block_k + (int64_t)a->block_k * a->block_n) * es;
+  const int64_t ring = (int64_t)a->num_stages * ((int64_t)a->block_m * a->block_k + (int64_t)a->block_k * a->block_n) * es;
+  // the epilogue passes the accumulators through per-wave LDS strips laid over the ring (EpiStage in
+  // gemm_tile.h): waves x MFMA rows x (wave-tile width x 4 bytes + 16).  Same wave grid as TileCfg.
+  const int nw = a->num_warps > 0 ? a->num_warps : 4;
+  const int wgm = nw == 4 ? 2 : (a->block_m > a->block_n ? 4 : 2), wgn = nw / wgm > 0 ? nw / wgm : 1;
+  const int wtm = a->block_m / wgm, wtn = a->block_n / wgn;
+  const int mi = (wtm % 32 == 0 && wtn % 32 == 0) ? 32 : 16;
+  const int64_t strips = (int64_t)nw * mi * (wtn * 4 + 16);
+  return ring > strips ? ring : strips;
 }
 
 static int check_common(const tnx_gemm_args* a) {
@@ -123,6 +131,7 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
   if (tiles * a->split_k > 0x7fffffffll) return TNX_E_UNSUPPORTED;
   if (cut_tiles(a) > WS_MAX_TILES) return TNX_E_UNSUPPORTED;  // one arrival counter per cut tile
+  if (tnx_gemm_workspace_bytes(a) >= (1ull << 32)) return TNX_E_UNSUPPORTED;  // slices are addressed with 32-bit offsets
   if (out) *out = e;
   if (fast) *fast = f;
   return TNX_OK;
@@ -192,8 +201,7 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   a->block_k = bk;
   bool dma_ok;
   {
-    tnx_gemm_args t = *a;
-    t.a = t.b = nullptr;
+    tnx_gemm_args t = *a;   // a and b, when given, count with their base alignment (null = aligned)
     if (t.stride_ak == 0 && t.stride_bn == 0) { t.stride_am = t.k; t.stride_ak = 1; t.stride_bk = t.n; t.stride_bn = 1; }
     t.block_m = 128; t.block_n = 128; t.block_k = bk;
     dma_ok = fast_layout(&t);

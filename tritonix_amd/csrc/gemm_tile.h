@@ -134,7 +134,7 @@ __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint3
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
-               : "memory");
+               : "memory", "m0");
 }
 
 // same, with the non-temporal hint: for an operand that is streamed from HBM once and never reused
@@ -142,7 +142,7 @@ __device__ __forceinline__ void dma16_nt(const uint8_t* sbase, uint32_t voff, ui
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
-               : "memory");
+               : "memory", "m0");
 }
 
 __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
@@ -151,21 +151,21 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
   return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
-// Device-scope (all XCDs) 16-byte accesses for data that workgroups hand to each other inside
-// one kernel: the sc1 bit writes through / reads around the per-XCD L2, so no whole-cache
-// write-back or invalidate is needed around them.  The load does not wait: loads_landed()
-// does, for all loads passed to it.
-__device__ __forceinline__ void store16_agent(void* dst, i32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
+// Device-scope (all XCDs) 16-byte accesses for data that workgroups hand to each other inside one kernel,
+// as raw buffer operations with the sc1 bit: on gfx942/gfx950 that is the encoding of a monotonic atomic
+// access at agent scope (the store writes through the XCD's L2, the load does not hit a stale line of it),
+// so no whole-cache write-back or invalidate is needed around them.  They are compiler builtins, so the
+// compiler itself places the s_waitcnt before the first use of a loaded value.
+constexpr int CPOL_SC1 = 16;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t agent_window(const void* base) {
+  // raw buffer (stride 0) of 4 GiB - 1 bytes starting at base; offsets are unsigned 32-bit
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
 }
-__device__ __forceinline__ void load16_agent_nowait(i32x4& v, const void* src) {
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(src) : "memory");
+__device__ __forceinline__ void store16_agent(__amdgpu_buffer_rsrc_t w, uint32_t off, i32x4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, w, off, 0, CPOL_SC1);
 }
-template <int N> __device__ __forceinline__ void loads_landed(i32x4 (&v)[N]) {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  // tie every loaded value to the wait, so that no use is scheduled above it
-#pragma unroll
-  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i]) : : "memory");
+__device__ __forceinline__ i32x4 load16_agent(__amdgpu_buffer_rsrc_t w, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(w, off, 0, CPOL_SC1);
 }
 
 template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
@@ -302,7 +302,7 @@ template <bool GLU> struct Pack16<int, int, GLU> {            // int32 outputs: 
 // instruction moves one contiguous KiB.
 struct SliceSrc {
   const uint8_t* base;     // this wave's part of slice 0
-  int64_t slice_stride;    // bytes from one slice to the next
+  uint32_t slice_stride;   // bytes from one slice to the next (the host keeps nslices * slice_stride under 4 GiB)
   int nslices;
 };
 
@@ -310,7 +310,8 @@ struct SliceSrc {
 // strip (same places the accumulators of an uncut tile go).  ZB slices of G = 32 / ZB groups
 // are fetched together; slices are added in slice order whatever ZB is.
 template <class ACC4, int ZB, int NQ, int MI, int NGRP>
-__device__ __forceinline__ void sum_slices(const uint8_t* q0, const SliceSrc& src, uint32_t wbase, bool row_ok) {
+__device__ __forceinline__ void sum_slices(__amdgpu_buffer_rsrc_t win, uint32_t q0, const SliceSrc& src, uint32_t wbase,
+                                           bool row_ok) {
   constexpr int G = (32 / ZB) < NQ ? (32 / ZB) : NQ;
   static_assert(NQ % G == 0, "groups per row-block must be a multiple of the batch");
 #pragma unroll 1
@@ -327,9 +328,8 @@ __device__ __forceinline__ void sum_slices(const uint8_t* q0, const SliceSrc& sr
 #pragma unroll
         for (int u = 0; u < ZB; ++u) {
           const int z = z0 + u < src.nslices ? z0 + u : src.nslices - 1;
-          load16_agent_nowait(w[x * ZB + u], q0 + (int64_t)(jg0 + x) * 1024 + z * src.slice_stride);
+          w[x * ZB + u] = load16_agent(win, q0 + (uint32_t)(jg0 + x) * 1024u + (uint32_t)z * src.slice_stride);
         }
-      loads_landed(w);
 #pragma unroll
       for (int x = 0; x < G; ++x)
 #pragma unroll
@@ -387,14 +387,15 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
               acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
     } else {
       // 32 loads per lane in flight (G groups x ZB slices): the hand-over is latency-bound otherwise
-      const uint8_t* q0 = src.base + (int64_t)i * (C::TN * NGRP) * 1024 + lane * 16;
+      const __amdgpu_buffer_rsrc_t win = agent_window(src.base);
+      const uint32_t q0 = (uint32_t)i * (C::TN * NGRP) * 1024u + lane * 16u;
       const bool row_ok = gm0 + i * MI + lane % MI < m;
       if (src.nslices <= 2)
-        sum_slices<acc4, 2, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+        sum_slices<acc4, 2, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
       else if (src.nslices <= 4)
-        sum_slices<acc4, 4, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+        sum_slices<acc4, 4, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
       else
-        sum_slices<acc4, 8, C::TN * NGRP, MI, NGRP>(q0, src, wbase, row_ok);
+        sum_slices<acc4, 8, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
     }
     // the strip is private to this wave: its own LDS writes are ordered before its reads
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
@@ -458,6 +459,7 @@ __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t*
   typedef acc_s acc4 __attribute__((ext_vector_type(4)));
   constexpr int NGRP = C::ACC_N / 4;
   constexpr int NQ = C::TN * NGRP;                      // 16-byte groups per lane and row-block
+  const __amdgpu_buffer_rsrc_t win = agent_window(wave_slice);
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
     if (gm0 + i * C::MI >= m) break;
@@ -470,10 +472,11 @@ __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t*
         *TNX_LDS(acc4, lds_strip + (j * NGRP + g) * 1024 + lane * 16) =
             acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    uint8_t* dst = wave_slice + (int64_t)i * NQ * 1024 + lane * 16;
+    const uint32_t dst = (uint32_t)i * NQ * 1024u + lane * 16u;
     if (gm0 + i * C::MI + lane % C::MI < m) {            // a lane is one row: rows past the problem are not stored
 #pragma unroll 4
-      for (int q = 0; q < NQ; ++q) store16_agent(dst + q * 1024, *TNX_LDS(i32x4, lds_strip + q * 1024 + lane * 16));
+      for (int q = 0; q < NQ; ++q)
+        store16_agent(win, dst + q * 1024u, *TNX_LDS(i32x4, lds_strip + q * 1024 + lane * 16));
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);
   }
@@ -839,7 +842,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     if (!splitk_arrive<T, C>(acc, wave0 + split * slice_stride, strip, lane, gm0, p.m, (int*)p.ws + ctile, (int*)smem,
                              p.split_k))
       return;
-    const SliceSrc src = {wave0, slice_stride, p.split_k};
+    const SliceSrc src = {wave0, (uint32_t)slice_stride, p.split_k};
     if (p.epilogue == EPI_NONE)
       epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
     else

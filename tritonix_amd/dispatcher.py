@@ -10,7 +10,10 @@ the JSON record ``{"op", "key", "winner", "timings"}`` in a file called
 ``backend_dispatch.json``.  Differences: records live under
 ``$TRITONIX_CACHE_DIR`` (default ``~/.cache/tritonix_amd``) rather than in
 Triton's cache, the timer is this package's HIP-event ``do_bench`` unless a
-``bench_fn`` is injected, and ``alias`` lets one backend answer to two names.
+``bench_fn`` is injected, ``alias`` lets one backend answer to two names, and a
+backend registered with ``raced=False`` is reachable through ``force_backend``
+only: it is never timed and never wins a signature (how ``torch.matmul`` stays
+available as the correctness oracle without ever serving an unforced call).
 """
 from __future__ import annotations
 
@@ -138,15 +141,25 @@ class DynamicDispatcher:
         self._bench_fn = bench_fn
         self._store = _RecordStore(self.__name__) if use_disk_cache else None
         self._backends: Dict[str, Callable] = {}
+        self._unraced: set = set()
         self._aliases: Dict[str, str] = {}
         self._forced: Optional[str] = None
         self.cache: Dict[tuple, str] = {}
         self.timings: Dict[tuple, Dict[str, float]] = {}
 
     # -- registration -------------------------------------------------------
-    def register(self, name: str, impl: Callable) -> "DynamicDispatcher":
+    def register(self, name: str, impl: Callable, raced: bool = True) -> "DynamicDispatcher":
+        """Add (or replace) a backend.  ``raced=False`` keeps it out of the timing race and out of ``cache``:
+        only ``force_backend(name)`` reaches it."""
         self._backends[name] = impl
+        if raced:
+            self._unraced.discard(name)
+        else:
+            self._unraced.add(name)
         return self
+
+    def _contenders(self) -> Dict[str, Callable]:
+        return {name: impl for name, impl in self._backends.items() if name not in self._unraced}
 
     def alias(self, alias: str, name: str) -> "DynamicDispatcher":
         """Make ``force_backend(alias)`` select backend ``name``; timings and records keep the one real name."""
@@ -176,7 +189,7 @@ class DynamicDispatcher:
         """Winner for a signature seen for the first time in this process: a record on disk, else a race."""
         names = list(self._backends)
         verdict = self._store.get(names, signature) if self._store else None
-        if verdict is None or verdict.winner not in self._backends:
+        if verdict is None or verdict.winner not in self._contenders():
             verdict = self._race(args, kwargs)
             if self._store:
                 self._store.put(names, signature, verdict)
@@ -184,12 +197,12 @@ class DynamicDispatcher:
         return verdict.winner
 
     def _race(self, args: tuple, kwargs: dict) -> _Verdict:
-        """Time every backend on this very call; one that raises simply does not finish."""
+        """Time every raced backend on this very call; one that raises simply does not finish."""
         clock = self._bench_fn
         if clock is None:
             from tritonix_amd.testing import do_bench as clock
         finished: Dict[str, float] = {}
-        for name, impl in self._backends.items():
+        for name, impl in self._contenders().items():
             try:
                 finished[name] = clock(lambda: impl(*args, **kwargs), **self._budget)
             except Exception as err:

@@ -14,8 +14,12 @@ Deliberate differences:
     LDS stages); a combination that is not built raises ``ValueError`` and the
     tuner skips it, one that exceeds 160 KiB of LDS raises ``OutOfResources``
     before any launch and the trie prunes above it;
-  * the config memo is keyed by dtype as well as (m, n, k), because one
-    process now runs f16, bf16 and int8 problems;
+  * the config memo is keyed by dtype and by the layout class of the operands
+    (row-major, 16-byte aligned rows and base pointers, or anything else) as
+    well as (m, n, k): one process runs f16, bf16 and int8 problems, and most
+    tiles exist only with the direct-to-LDS loader that needs the first class;
+  * ``matmul`` races HIP variants only (tuned tile, split-K, the 16-row
+    kernel); ``torch.matmul`` is registered un-raced, for ``force_backend``;
   * int8 inputs give an int32 result;
   * split-K sums fp32 partials from a workspace and rounds once, where the
     reference rounds each partial to the output dtype and adds atomically
@@ -31,7 +35,8 @@ from tritonix_amd.autotune import Choice, PowerOfTwo, Range, tunable
 from tritonix_amd.dispatcher import dynamic_dispatch
 from tritonix_amd.kernel import HipKernel, cdiv, out_dtype_for
 
-__all__ = ["matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel", "gemm_splitk_kernel",
+__all__ = ["matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_skinny", "matmul_kernel", "gemm_splitk_kernel",
+           "dma_layout", "run_memoised",
            "swizzle2d", "grouped_launch", "TUNE_OPTIONS", "load_tuned", "save_tuned"]
 
 # keyword arguments handed to ``.tune`` on a config-memo miss (tests shrink the time budgets)
@@ -170,6 +175,15 @@ def save_tuned(op: str, key: tuple, cfg: dict) -> None:
         pass
 
 
+def dma_layout(a, b) -> bool:
+    """True when the operands can take the direct-to-LDS loader: row-major A and B, 16-byte aligned rows and base
+    pointers.  Most tile kernels are built with that loader only, so it is part of every config-memo key."""
+    es = a.element_size()
+    return bool(a.stride(1) == 1 and b.stride(1) == 1 and a.stride(0) >= 0 and b.stride(0) >= 0
+                and (a.stride(0) * es) % 16 == 0 and (b.stride(0) * es) % 16 == 0
+                and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0 and b.shape[1] % (16 // es) == 0)
+
+
 def _tuned_or_tune(op: str, key: tuple, kernel, launcher, fallback):
     """Config for ``key``: disk record, else a grid search (stored afterwards), else the built-in choice."""
     if not _autotune_enabled():
@@ -188,6 +202,21 @@ def _tuned_or_tune(op: str, key: tuple, kernel, launcher, fallback):
     return cfg
 
 
+def run_memoised(memo: dict, op: str, key: tuple, kernel, launcher, fallback):
+    """Launch with the config remembered for ``key`` (finding one first if there is none).
+
+    A remembered config that the engine refuses for these very operands (``ValueError``: the layout changed in a
+    way the key does not capture, or the memo was filled by hand) is replaced by the built-in choice for them.
+    """
+    if key not in memo:
+        memo[key] = _tuned_or_tune(op, key, kernel, launcher, fallback)
+    try:
+        return launcher(memo[key])
+    except ValueError:
+        memo[key] = fallback()
+        return launcher(memo[key])
+
+
 def default_config(a, b, split=False):
     """The engine's built-in tile choice for this problem (used when tuning is switched off)."""
     import ctypes
@@ -201,6 +230,9 @@ def default_config(a, b, split=False):
     g.stride_am, g.stride_ak = a.stride()
     g.stride_bk, g.stride_bn = b.stride()
     g.in_dtype = _torch_dtype_code(a.dtype)
+    # base-pointer alignment decides between the two loaders; CPU tensors (host-side planning) count as aligned
+    g.a = a.data_ptr() if a.is_cuda else None
+    g.b = b.data_ptr() if b.is_cuda else None
     _C.load().tnx_gemm_default_config(ctypes.byref(g))
     cfg = {"block_m": g.block_m, "block_n": g.block_n, "block_k": g.block_k, "group_m": g.group_m,
            "num_stages": g.num_stages, "num_warps": g.num_warps}
@@ -219,7 +251,7 @@ def _autotune_enabled() -> bool:
 
 
 def triton_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """C = A @ B on the HIP tile kernel, tile config tuned once per (m, n, k, dtype).
+    """C = A @ B on the HIP tile kernel, tile config tuned once per (m, n, k, dtype, layout class).
 
     Keeps the reference's name: callers and the ``"triton"`` backend label of
     ``matmul`` refer to it.  ``hip_matmul`` is the same function.
@@ -227,11 +259,9 @@ def triton_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     _check_2d(a, b)
     m, k = a.shape
     _, n = b.shape
-    key = (m, n, k, a.dtype)
-    if key not in _matmul_cfg:
-        _matmul_cfg[key] = _tuned_or_tune("matmul", key, matmul_kernel, lambda cfg: _launch_matmul(a, b, cfg),
-                                          lambda: default_config(a, b))
-    return _launch_matmul(a, b, _matmul_cfg[key])
+    key = (m, n, k, a.dtype, dma_layout(a, b))
+    return run_memoised(_matmul_cfg, "matmul", key, matmul_kernel, lambda cfg: _launch_matmul(a, b, cfg),
+                        lambda: default_config(a, b))
 
 
 hip_matmul = triton_matmul
@@ -246,13 +276,35 @@ def matmul_splitk(a: torch.Tensor, b: torch.Tensor, split_k: int = 4) -> torch.T
     _check_2d(a, b)
     m, k = a.shape
     _, n = b.shape
-    key = (m, n, k, split_k, a.dtype)
-    if key not in _splitk_cfg:
-        _splitk_cfg[key] = _tuned_or_tune("matmul_splitk", key, gemm_splitk_kernel,
-                                          lambda cfg: _launch_splitk(a, b, cfg),
-                                          lambda: default_config(a, b, split=True))
-    return _launch_splitk(a, b, _splitk_cfg[key])
+    key = (m, n, k, split_k, a.dtype, dma_layout(a, b))
+    return run_memoised(_splitk_cfg, "matmul_splitk", key, gemm_splitk_kernel, lambda cfg: _launch_splitk(a, b, cfg),
+                        lambda: default_config(a, b, split=True))
 
 
-matmul = dynamic_dispatch({"triton": triton_matmul, "pytorch": torch.matmul}, key=["a", "b"])
+# the m <= 16 kernel: eight waves of a workgroup each take an eighth of K and meet in LDS
+SKINNY_CONFIG = {"block_m": 16, "block_n": 32, "block_k": 32, "group_m": 8, "split_k": 8, "num_stages": 4,
+                 "num_warps": 8}
+
+
+def matmul_skinny(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """C = A @ B for at most 16 rows on the wavefront-level split-K kernel; ``ValueError`` for any other shape."""
+    _check_2d(a, b)
+    return _launch_splitk(a, b, SKINNY_CONFIG)
+
+
+def _splitk_backend(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``matmul_splitk`` as a contender of the dispatcher: only for problems whose output tiles alone leave CUs
+    idle (fewer 64x128 tiles than the part has CUs); any other problem drops out of the race."""
+    _check_2d(a, b)
+    if cdiv(a.shape[0], 64) * cdiv(b.shape[1], 128) >= 256:
+        raise ValueError("the output tiles fill the CUs: no K split is raced for this shape")
+    return matmul_splitk(a, b)
+
+
+# The dispatcher selects among HIP variants only.  ``torch.matmul`` (the reference's "pytorch" backend,
+# tritonix/ops/matmul.py:291-293) is the correctness oracle: ``force_backend("pytorch")`` reaches it, the race
+# never does, so an unforced ``matmul(a, b)`` always runs a kernel of this library.
+matmul = dynamic_dispatch({"triton": triton_matmul, "splitk": _splitk_backend, "skinny": matmul_skinny},
+                          key=["a", "b"])
+matmul.register("pytorch", torch.matmul, raced=False)
 matmul.alias("hip", "triton")

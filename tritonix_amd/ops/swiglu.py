@@ -76,11 +76,9 @@ def glu(x: torch.Tensor, w12: torch.Tensor, activation: str = "silu") -> torch.T
         raise ValueError(f"glu is built for float16 and bfloat16, got {x.dtype}")
     m, k = x.shape
     n = w12.shape[1]
-    key = (m, n, k, x.dtype)
-    if key not in _glu_cfg:
-        _glu_cfg[key] = _mm._tuned_or_tune("glu", key, glu_kernel, lambda cfg: _launch_glu(x, w12, cfg, activation),
-                                           lambda: _mm.default_config(x, w12))
-    return _launch_glu(x, w12, _glu_cfg[key], activation)
+    key = (m, n, k, x.dtype, _mm.dma_layout(x, w12))
+    return _mm.run_memoised(_glu_cfg, "glu", key, glu_kernel, lambda cfg: _launch_glu(x, w12, cfg, activation),
+                            lambda: _mm.default_config(x, w12))
 
 
 def swiglu(x: torch.Tensor, w12: torch.Tensor) -> torch.Tensor:
