@@ -57,7 +57,8 @@ enum tnx_status {
   TNX_E_UNSUPPORTED = 2, /* no kernel is built for this tile / dtype / layout combo   */
   TNX_E_LDS = 3,         /* the tile config needs more LDS than one CU has            */
   TNX_E_WORKSPACE = 4,   /* split_k > 1 and the workspace is missing or too small     */
-  TNX_E_HIP = 5          /* the HIP runtime reported an error (see tnx_last_hip_error) */
+  TNX_E_HIP = 5,         /* the HIP runtime reported an error (see tnx_last_hip_error) */
+  TNX_E_STATIC_LIMIT = 6 /* tnx_gemm_static_workspace: the launch needs more scratch than the static buffer */
 };
 
 /* Per-CU LDS capacity on gfx950; the budget tile configs are pruned against. */
@@ -94,6 +95,20 @@ typedef struct tnx_gemm_args {
 
 /* Launch one GEMM.  Returns a tnx_status.  Asynchronous. */
 int tnx_gemm(const tnx_gemm_args* args);
+
+/* tnx_gemm without any allocation on anyone's side.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory at the call site (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  Same arguments and results as tnx_gemm, except that
+ * `workspace` / `workspace_bytes` are ignored: a split-K launch takes its scratch from a buffer of
+ * TNX_STATIC_WORKSPACE_BYTES that is part of the library's device image (every GPU the library runs
+ * on holds one copy until the process ends).  A launch that needs more returns TNX_E_STATIC_LIMIT and
+ * launches nothing.  The call makes no hipMalloc / hipFree and calls no allocating routine; it enqueues
+ * one extra tiny kernel that clears the arrival counters it is about to use.  All calls on one GPU share
+ * that GPU's buffer: calls that may overlap on one GPU (different streams, or different threads) race
+ * and must be ordered by the caller.  The first call on a device looks the buffer's address up
+ * (hipGetSymbolAddress) and must therefore happen outside graph capture. */
+#define TNX_STATIC_WORKSPACE_BYTES (65536 + (32 << 20))
+int tnx_gemm_static_workspace(const tnx_gemm_args* args);
 
 /* Bytes of device scratch tnx_gemm needs for these args (0 when split_k <= 1):
  * the counters plus split_k fp32/int32 copies of every tile that is cut.

@@ -19,9 +19,10 @@ F16, BF16, I8, I32, F32 = 0, 1, 2, 3, 4
 # enum tnx_epilogue
 EPI_NONE, EPI_GLU_SILU, EPI_GLU_SIGMOID, EPI_GLU_IDENTITY = 0, 1, 2, 3
 # enum tnx_status
-OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP = 0, 1, 2, 3, 4, 5
+OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP, E_STATIC_LIMIT = 0, 1, 2, 3, 4, 5, 6
+STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
 
-EXPORTS = ("tnx_gemm", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
+EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
            "tnx_gemm_default_config", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
            "tnx_last_hip_error", "tnx_version")
 
@@ -59,6 +60,8 @@ def load() -> ctypes.CDLL:
     p = ctypes.POINTER(GemmArgs)
     lib.tnx_gemm.argtypes = [p]
     lib.tnx_gemm.restype = ctypes.c_int
+    lib.tnx_gemm_static_workspace.argtypes = [p]
+    lib.tnx_gemm_static_workspace.restype = ctypes.c_int
     lib.tnx_gemm_workspace_bytes.argtypes = [p]
     lib.tnx_gemm_workspace_bytes.restype = ctypes.c_size_t
     lib.tnx_gemm_lds_bytes.argtypes = [p]
@@ -98,7 +101,7 @@ def raise_for_status(status: int, args: GemmArgs) -> None:
             f"warps={args.num_warps} stages={args.num_stages} split_k={args.split_k} epilogue={args.epilogue}")
     if status == E_HIP:
         raise RuntimeError(f"{strerror(status)} (hipError_t {lib.tnx_last_hip_error()})")
-    if status == E_WORKSPACE:
+    if status in (E_WORKSPACE, E_STATIC_LIMIT):
         raise RuntimeError(strerror(status))
     raise ValueError(strerror(status))
 

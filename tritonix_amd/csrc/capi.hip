@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "../../include/tritonix_hip.h"
 #include "registry.h"
 
@@ -190,6 +192,66 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   return TNX_OK;
 }
 
+// ---------------------------------------------------------------------------
+// tnx_gemm_static_workspace: the split-K scratch lives in a file-scope device array instead of a
+// caller-provided workspace, so the call allocates nothing.  `scratch` is a host-side handle here:
+// the device address is looked up once per device with hipGetSymbolAddress and only that pointer
+// is ever handed to kernels.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[TNX_STATIC_WORKSPACE_BYTES];
+
+static constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+__global__ void zero_words_kernel(int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// device address of this device's copy of `scratch` (each GPU holds its own copy at its own address)
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+  if (dev < 0 || dev >= MAX_DEVICES) return TNX_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return TNX_OK;
+}
+
+extern "C" int tnx_gemm_static_workspace(const tnx_gemm_args* a) {
+  if (!a) return TNX_E_INVALID;
+  tnx_gemm_args t = *a;
+  t.workspace = nullptr;
+  t.workspace_bytes = 0;
+  const size_t need = tnx_gemm_workspace_bytes(&t);
+  if (need > 0) {
+    if (need > (size_t)TNX_STATIC_WORKSPACE_BYTES) return TNX_E_STATIC_LIMIT;
+    int st = supported_impl(&t, nullptr, nullptr, true);
+    if (st != TNX_OK) return st;
+    void* ptr = nullptr;
+    st = scratch_of_current_device(&ptr);
+    if (st != TNX_OK) return st;
+    // The array keeps what the last call left.  The arrival counters of the tiles this launch cuts must
+    // start at zero; a launch leaves them zero, but one that was aborted does not, so they are cleared
+    // here with a small fill kernel (legal under graph capture, unlike a memset node).
+    const int words = (int)cut_tiles(&t);
+    hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)t.stream, (int*)ptr, words);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+    t.workspace = ptr;
+    t.workspace_bytes = TNX_STATIC_WORKSPACE_BYTES;
+  }
+  return tnx_gemm(&t);
+}
+
 extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   if (!a) return TNX_E_INVALID;
   const int es = elem_size(a->in_dtype);
@@ -293,6 +355,7 @@ extern "C" const char* tnx_strerror(int status) {
     case TNX_E_LDS: return "tile configuration exceeds the per-CU LDS budget";
     case TNX_E_WORKSPACE: return "split-K workspace missing or too small";
     case TNX_E_HIP: return "HIP runtime error";
+    case TNX_E_STATIC_LIMIT: return "split-K scratch of this launch exceeds TNX_STATIC_WORKSPACE_BYTES (use tnx_gemm with a workspace)";
     default: return "unknown status";
   }
 }
