@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the tiled-GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune] [--only C2,C5] [--operands random|zeros]
+                    [--sustain SECONDS] [--no-extras] [--no-cpu] [--no-vendor]
 
 A step is one launch of the headline workload -- the bf16 8192^3 GEMM
 (row-major A and B, fp32 accumulate, bf16 out, non-split tiled kernel with
@@ -9,27 +10,42 @@ the group-M swizzle) -- through the C ABI, operands resident in HBM.  Prints
 one JSON line: whole-job TFLOP/s over the K timed steps, the roofline record
 of the kernel (algorithmic flops / mean per-launch duration from HIP events
 on the launch stream), the CPU baseline (torch fp32 matmul on the host
-cores, bounded sample) and, under "per_config", the other four benchmark
+cores, bounded sample) and, under "per_config", the other benchmark
 configurations measured the same way.  "vendor_ms" entries time torch's own
 GPU matmul (rocBLAS / hipBLASLt) on the same operands in the same run, for
 comparison only: nothing in the measured path calls it.
+
+Switches for profiling and for the clock / power evidence:
+  --only C2,C5       run these workloads only (the headline C2 is always what `value` reports when it is run;
+                     without it the line carries per_config only and `value` is null)
+  --operands zeros   all-zero operands of the same shapes: the same instruction stream without data-dependent
+                     switching power, so the shader clock stays at its maximum (results are then trivially zero)
+  --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
+                     socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import subprocess
 import sys
+import threading
 import time
 
 PEAK = {"bf16": 2516.6, "f16": 2516.6, "i8": 5033.2}     # dense MFMA TFLOP/s (TOP/s), MI355X
 HBM_PEAK_GBS = 8000.0
 PRE_ROLL = 40                                            # untimed launches that bring the part out of idle clocks
+NOMINAL_SCLK_MHZ = 2400.0
 
 # L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
-# (KiB per dispatch), each scaled by what the same counter reads for bench.py's 2^28-byte calibration pass:
-# (844109.5 * 2.0 + 131072.0 * 1.0) KiB.  See profiles/gemm_tile_bf16_256x256x64_w4_c2_8192.md.
-TRAFFIC_BYTES_C2 = int((844109.5 * 2.0 + 131072.0 * 1.0) * 1024)
+# (KiB per dispatch), each scaled by what the same counter reads for this file's 2^28-byte calibration pass.
+# The two readings and the two factors are in profiles/gemm_tile_bf16_256x256x64_c2_counters.md.
+TRAFFIC_KIB_C2 = {"fetch": 844109.5, "fetch_scale": 2.0, "write": 131072.0, "write_scale": 1.0}
+TRAFFIC_BYTES_C2 = int((TRAFFIC_KIB_C2["fetch"] * TRAFFIC_KIB_C2["fetch_scale"]
+                        + TRAFFIC_KIB_C2["write"] * TRAFFIC_KIB_C2["write_scale"]) * 1024)
+
+ALL = ("C2", "C1", "C3", "C4", "C5", "FFN")
 
 
 def parse():
@@ -38,6 +54,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--tune", action="store_true", help="run the grid tuner for each workload instead of the built-in tiles")
+    ap.add_argument("--only", default=None, help="comma-separated subset of " + ",".join(ALL))
+    ap.add_argument("--operands", choices=("random", "zeros"), default="random")
+    ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocBLAS/hipBLASLt timing of the same operands")
@@ -103,6 +122,65 @@ def pick_config(kernel, launcher, a, b, tune, split=False):
     return default_config(a, b, split=split)
 
 
+def smi_sample():
+    """(socket power in W, shader clock in MHz) from `amd-smi metric -p -c --json`, or None."""
+    try:
+        out = subprocess.run(["amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True, timeout=10).stdout
+        gpu = json.loads(out)["gpu_data"][0]
+        clocks = [v["clk"]["value"] for k, v in gpu["clock"].items() if k.startswith("gfx_") and isinstance(v.get("clk"), dict)]
+        return float(gpu["power"]["socket_power"]["value"]), float(sum(clocks) / len(clocks))
+    except Exception:
+        return None
+
+
+def power_limit_w():
+    try:
+        out = subprocess.run(["rocm-smi", "-M", "--json"], capture_output=True, text=True, timeout=10).stdout
+        card = next(iter(json.loads(out).values()))
+        return float(next(v for k, v in card.items() if "Max Graphics Package Power" in k))
+    except Exception:
+        return None
+
+
+def sustain(step, seconds, flops):
+    """Launch `step` continuously for `seconds`; a second thread samples power and clock meanwhile.
+
+    The first second of samples is dropped (the management firmware reports moving averages)."""
+    import torch
+
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            s = smi_sample()
+            if s is not None:
+                samples.append((time.perf_counter(), *s))
+
+    th = threading.Thread(target=poll, daemon=True)
+    t0 = time.perf_counter()
+    th.start()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(200):
+            step()
+        torch.cuda.synchronize()
+        n += 200
+    elapsed = time.perf_counter() - t0
+    stop.set()
+    th.join(timeout=15)
+    kept = [(p, c) for t, p, c in samples if t - t0 > 1.0 and t - t0 < elapsed]
+    out = {"seconds": round(elapsed, 2), "launches": n, "tflops": round(flops * n / elapsed / 1e12, 1),
+           "samples": len(kept), "power_limit_w": power_limit_w()}
+    if kept:
+        pw, ck = [p for p, _ in kept], [c for _, c in kept]
+        out.update({"socket_power_w_mean": round(sum(pw) / len(pw), 1), "socket_power_w_max": max(pw),
+                    "sclk_mhz_mean": round(sum(ck) / len(ck), 1), "sclk_mhz_min": min(ck), "sclk_mhz_max": max(ck)})
+        # what a kernel that kept every MFMA pipe busy in every cycle would reach at the clock the part actually ran
+        out["mfma_peak_at_sclk_tflops"] = round(PEAK["bf16"] * out["sclk_mhz_mean"] / NOMINAL_SCLK_MHZ, 1)
+        out["mfma_busy_at_sclk"] = round(out["tflops"] / out["mfma_peak_at_sclk_tflops"], 4)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -128,6 +206,20 @@ def main():
     _C.load()
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    only = tuple(s.strip() for s in args.only.split(",")) if args.only else ALL
+    unknown = [s for s in only if s not in ALL]
+    if unknown:
+        print(f"unknown workload(s) {unknown}; choose from {ALL}", file=sys.stderr)
+        return 2
+    if args.no_extras:
+        only = tuple(s for s in only if s == "C2")
+    zeros = args.operands == "zeros"
+
+    def operands(name):
+        a, b = oracle.make_inputs(name)
+        if zeros:
+            a, b = torch.zeros_like(a), torch.zeros_like(b)
+        return a, b
 
     # one plain elementwise pass of known size (2^28 bytes read, 2^28 bytes written): under
     # `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` it is the dispatch the GEMM's counter readings are scaled by
@@ -137,8 +229,24 @@ def main():
     torch.cuda.synchronize()
     del cal_src, cal_dst
 
-    # ---- headline: C2 --------------------------------------------------------------
-    a_cpu, b_cpu = oracle.make_inputs("C2")
+    out = {
+        "metric": "TFLOP/s + % of dense MFMA peak, bf16 GEMM 8192³ on 1×MI355X",
+        "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic" if not zeros else "synthetic (all-zero operands: clock evidence, not a result)",
+    }
+    ok = True
+    if "C2" in only:
+        ok = headline(torch, dev, oracle, mm, args, operands, out)
+    extras_wanted = [s for s in only if s != "C2"]
+    if extras_wanted:
+        out["per_config"] = extras(torch, dev, oracle, mm, sg, args, operands, extras_wanted)
+    print(json.dumps(out))
+    return 0 if ok else 1
+
+
+def headline(torch, dev, oracle, mm, args, operands, out):
+    a_cpu, b_cpu = operands("C2")
     a, b = a_cpu.to(dev), b_cpu.to(dev)
     m, k = a.shape
     n = b.shape[1]
@@ -148,7 +256,6 @@ def main():
         bm, bn, bk, nw, st, gm = (int(v) for v in args.tile.split(","))
         cfg = {"block_m": bm, "block_n": bn, "block_k": bk, "group_m": gm, "num_stages": st, "num_warps": nw}
     c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
-    grid = (-(-m // cfg["block_m"]), -(-n // cfg["block_n"]))
 
     # one C-ABI call per step: the arguments are bound once, the step is `tnx_gemm(&args)`
     launch = mm.matmul_kernel.prepare(a, b, c, m, n, k, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0),
@@ -193,6 +300,8 @@ def main():
     rows = torch.arange(0, m, 517)
     ok, maxerr, rel = oracle.within_tolerance(c[rows.to(dev)], oracle.reference_matmul(a_cpu[rows], b_cpu))
 
+    sustained = sustain(step, args.sustain, flops) if args.sustain > 0 else None
+
     # ---- CPU baseline: the reference's "pytorch" backend restated on the host ---------
     cpu = None
     if not args.no_cpu:
@@ -212,31 +321,23 @@ def main():
         cpu = {"value": round(2.0 * rows_n * n * k / med / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
                "kind": "port", "sample": f"torch fp32 CPU matmul, first {rows_n} of {m} rows of A x full B, median of {reps}"}
 
-    out = {
-        "metric": "TFLOP/s + % of dense MFMA peak, bf16 GEMM 8192\u00b3 on 1\u00d7MI355X",
-        "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+    out.update({
+        "value": round(value, 1), "ms_per_step": round(ms_per_step, 4),
         "config": {"workload": "C2: bf16 GEMM M=N=K=8192, A,B ~ N(0,1)/sqrt(K) seed 2, row-major, fp32 acc, bf16 out",
-                   "tile": cfg},
+                   "tile": cfg, "operands": args.operands},
         "pct_of_peak": round(100 * value / PEAK["bf16"], 2),
         "roofline": roofline, "cpu_baseline": cpu, "vendor_blas": vendor,
         "parity": {"ok": bool(ok), "max_abs_err": maxerr, "max_err_over_max_ref": rel, "rows_checked": int(rows.numel())},
-    }
-    del a, b, c
-
-    # ---- the other configurations ------------------------------------------------------
-    if not args.no_extras:
-        out["per_config"] = extras(torch, dev, oracle, mm, sg, args)
-    print(json.dumps(out))
-    return 0 if ok else 1
+    })
+    if sustained is not None:
+        out["sustain"] = sustained
+    return ok
 
 
-def extras(torch, dev, oracle, mm, sg, args):
-    from tritonix_amd.kernel import out_dtype_for
-
+def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
     res = {}
     reps = 30
+    zeros = args.operands == "zeros"
 
     def measure(name, fn, flops, bytes_, dt, bound, nrot=1):
         for i in range(PRE_ROLL):
@@ -255,97 +356,129 @@ def extras(torch, dev, oracle, mm, sg, args):
         return r
 
     # C1: latency-bound, report only
-    a, b = (t.to(dev) for t in oracle.make_inputs("C1"))
-    cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
-    c = torch.empty((1024, 768), device=dev, dtype=torch.float16)
-    l1 = mm.matmul_kernel.prepare(a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg)
-    r = measure("C1", lambda i: l1(), 805306368, 3407872, "f16", None)
-    r["tile"] = cfg
-    if not args.no_vendor:
-        cv = torch.empty_like(c)
-        r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, b, out=cv))
-    if not args.no_cpu:
-        af, bf = a.cpu().float(), b.cpu().float()
-        t, n = cpu_time(lambda: torch.matmul(af, bf))
-        r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(805306368 / t / 1e9, 1), "cores": torch.get_num_threads(),
-                    "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
+    if "C1" in wanted:
+        a, b = (t.to(dev) for t in operands("C1"))
+        cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+        c = torch.empty((1024, 768), device=dev, dtype=torch.float16)
+        l1 = mm.matmul_kernel.prepare(a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg)
+        r = measure("C1", lambda i: l1(), 805306368, 3407872, "f16", None)
+        r["tile"] = cfg
+        if not args.no_vendor:
+            cv = torch.empty_like(c)
+            r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, b, out=cv))
+        if not args.no_cpu:
+            af, bf = a.cpu().float(), b.cpu().float()
+            t, n = cpu_time(lambda: torch.matmul(af, bf))
+            r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(805306368 / t / 1e9, 1), "cores": torch.get_num_threads(),
+                        "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
 
     # C3: B is streamed from HBM: rotate distinct copies of B so that none is served from the 256 MiB Infinity Cache
-    a_cpu, b_cpu = oracle.make_inputs("C3")
-    a = a_cpu.to(dev)
-    nrot = 4
-    bs = [b_cpu.to(dev).clone() for _ in range(nrot)]
-    cfg = pick_config(mm.gemm_splitk_kernel, lambda c: mm._launch_splitk(a, bs[0], c), a, bs[0], args.tune, split=True)
-    c = torch.empty((16, 4096), device=dev, dtype=torch.bfloat16)
-    l3 = [mm.gemm_splitk_kernel.prepare(a, bs[i], c, 16, 4096, 14336, 14336, 1, 4096, 1, 4096, 1, **cfg)
-          for i in range(nrot)]
-    r = measure("C3", lambda i: l3[i](), 1879048192, 118030336, "bf16", "hbm", nrot=nrot)
-    r["tile"] = cfg
-    r["note"] = f"{nrot} distinct copies of B rotated ({nrot * 117} MB > 256 MB Infinity Cache); one kernel, reduction fused"
-    ok, _, rel = oracle.within_tolerance(c, oracle.reference_matmul(a_cpu, b_cpu))
-    r["parity_ok"] = bool(ok)
-    if not args.no_vendor:
-        cv = torch.empty_like(c)
-        r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, bs[i % nrot], out=cv), reps=reps)
-    if not args.no_cpu:
-        af, bf = a_cpu.float(), b_cpu.float()
-        t, n = cpu_time(lambda: torch.matmul(af, bf))
-        r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(1879048192 / t / 1e9, 1), "cores": torch.get_num_threads(),
-                    "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
-        del af, bf
-    del bs
+    if "C3" in wanted:
+        a_cpu, b_cpu = operands("C3")
+        a = a_cpu.to(dev)
+        nrot = 4
+        bs = [b_cpu.to(dev).clone() for _ in range(nrot)]
+        cfg = pick_config(mm.gemm_splitk_kernel, lambda c: mm._launch_splitk(a, bs[0], c), a, bs[0], args.tune, split=True)
+        c = torch.empty((16, 4096), device=dev, dtype=torch.bfloat16)
+        l3 = [mm.gemm_splitk_kernel.prepare(a, bs[i], c, 16, 4096, 14336, 14336, 1, 4096, 1, 4096, 1, **cfg)
+              for i in range(nrot)]
+        r = measure("C3", lambda i: l3[i](), 1879048192, 118030336, "bf16", "hbm", nrot=nrot)
+        r["tile"] = cfg
+        r["note"] = f"{nrot} distinct copies of B rotated ({nrot * 117} MB > 256 MB Infinity Cache); one kernel, reduction fused"
+        okc, _, _ = oracle.within_tolerance(c, oracle.reference_matmul(a_cpu, b_cpu))
+        r["parity_ok"] = bool(okc)
+        if not args.no_vendor:
+            cv = torch.empty_like(c)
+            r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, bs[i % nrot], out=cv), reps=reps)
+        if not args.no_cpu:
+            af, bf = a_cpu.float(), b_cpu.float()
+            t, n = cpu_time(lambda: torch.matmul(af, bf))
+            r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(1879048192 / t / 1e9, 1), "cores": torch.get_num_threads(),
+                        "sample": f"torch fp32 CPU matmul, whole problem, median of {n}"}
+            del af, bf
+        del bs
 
-    # C4: fused GLU, both activations
-    x_cpu, w_cpu = oracle.make_inputs("C4")
-    x, w = x_cpu.to(dev), w_cpu.to(dev)
-    cfg = pick_config(sg.glu_kernel, lambda c: sg._launch_glu(x, w, c, "silu"), x, w, args.tune)
-    z = torch.empty((4096, 14336), device=dev, dtype=torch.bfloat16)
-    for act in ("silu", "sigmoid"):
-        l4 = sg.glu_kernel.prepare(x, w, z, 4096, 28672, 4096, 4096, 1, 28672, 1, 14336, 1, activation=act, **cfg)
-        measure(f"C4_{act}", lambda i: l4(), 962072674304, 385875968, "bf16", "mfma")["tile"] = cfg
-    rows = torch.arange(0, 4096, 409)
-    res["C4_sigmoid"]["parity_ok"] = bool(oracle.within_tolerance(z[rows.to(dev)],
-                                                                  oracle.reference_glu(x_cpu[rows], w_cpu, "sigmoid"))[0])
-    if not args.no_vendor:
-        g1 = torch.empty((4096, 28672), device=dev, dtype=torch.bfloat16)
-        res["C4_silu"]["vendor_ms"] = vendor_ms(lambda i: torch.matmul(x, w, out=g1))
-        res["C4_silu"]["vendor_note"] = "the [4096,28672] GEMM alone; gating would be a second pass over its output"
-        del g1
-    if not args.no_cpu:
-        import torch.nn.functional as F
+    # C4: fused GLU, both activations; FFN: the same up-projection followed by the down-projection (two launches)
+    if "C4" in wanted or "FFN" in wanted:
+        x_cpu, w_cpu = operands("C4")
+        x, w = x_cpu.to(dev), w_cpu.to(dev)
+        cfg = pick_config(sg.glu_kernel, lambda c: sg._launch_glu(x, w, c, "silu"), x, w, args.tune)
+        z = torch.empty((4096, 14336), device=dev, dtype=torch.bfloat16)
+        if "C4" in wanted:
+            for act in ("silu", "sigmoid"):
+                l4 = sg.glu_kernel.prepare(x, w, z, 4096, 28672, 4096, 4096, 1, 28672, 1, 14336, 1, activation=act, **cfg)
+                measure(f"C4_{act}", lambda i: l4(), 962072674304, 385875968, "bf16", "mfma")["tile"] = cfg
+            rows = torch.arange(0, 4096, 409)
+            res["C4_sigmoid"]["parity_ok"] = bool(oracle.within_tolerance(
+                z[rows.to(dev)], oracle.reference_glu(x_cpu[rows], w_cpu, "sigmoid"))[0])
+            if not args.no_vendor:
+                g1 = torch.empty((4096, 28672), device=dev, dtype=torch.bfloat16)
+                res["C4_silu"]["vendor_ms"] = vendor_ms(lambda i: torch.matmul(x, w, out=g1))
+                res["C4_silu"]["vendor_note"] = "the [4096,28672] GEMM alone; gating would be a second pass over its output"
+                del g1
+            if not args.no_cpu:
+                import torch.nn.functional as F
 
-        nr = 256
-        xf, w1, w2 = x_cpu[:nr].float(), w_cpu[:, 0::2].float(), w_cpu[:, 1::2].float()
-        t, n = cpu_time(lambda: F.silu(xf @ w1) * (xf @ w2))
-        res["C4_silu"]["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(962072674304 * nr / 4096 / t / 1e9, 1),
-                                 "cores": torch.get_num_threads(),
-                                 "sample": f"torch fp32 CPU silu(x@W1)*(x@W2), first {nr} of 4096 rows, median of {n}"}
-        del xf, w1, w2
-    del x, w, z
+                nr = 256
+                xf, w1, w2 = x_cpu[:nr].float(), w_cpu[:, 0::2].float(), w_cpu[:, 1::2].float()
+                t, n = cpu_time(lambda: F.silu(xf @ w1) * (xf @ w2))
+                res["C4_silu"]["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(962072674304 * nr / 4096 / t / 1e9, 1),
+                                         "cores": torch.get_num_threads(),
+                                         "sample": f"torch fp32 CPU silu(x@W1)*(x@W2), first {nr} of 4096 rows, median of {n}"}
+                del xf, w1, w2
+        if "FFN" in wanted:
+            # the SwiGLU feed-forward block at this size: silu-GLU up-projection [4096,4096]x[4096,28672] -> [4096,14336],
+            # then the down-projection [4096,14336]x[14336,4096]; the intermediate stays in HBM in bf16
+            g = torch.Generator("cpu").manual_seed(44)
+            w3_cpu = (0.02 * torch.randn(14336, 4096, generator=g)).bfloat16()
+            if zeros:
+                w3_cpu.zero_()
+            w3 = w3_cpu.to(dev)
+            y = torch.empty((4096, 4096), device=dev, dtype=torch.bfloat16)
+            cfg_d = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(z, w3, c), z, w3, args.tune)
+            up = sg.glu_kernel.prepare(x, w, z, 4096, 28672, 4096, 4096, 1, 28672, 1, 14336, 1, activation="silu", **cfg)
+            down = mm.matmul_kernel.prepare(z, w3, y, 4096, 4096, 14336, 14336, 1, 4096, 1, 4096, 1, **cfg_d)
+
+            def ffn(_i):
+                up()
+                down()
+
+            flops_ffn = 962072674304 + 2.0 * 4096 * 4096 * 14336
+            bytes_ffn = 385875968 + 2 * (4096 * 14336 + 14336 * 4096 + 4096 * 4096)
+            r = measure("FFN", ffn, flops_ffn, bytes_ffn, "bf16", "mfma")
+            r["tiles"] = {"up": cfg, "down": cfg_d}
+            r["note"] = ("swiglu_ffn = fused GLU up-projection + tiled GEMM down-projection, two launches; the [4096,14336] "
+                         "bf16 intermediate (117 MB) is written and read back once")
+            rows = torch.arange(0, 4096, 585)
+            hidden = oracle.reference_glu(x_cpu[rows], w_cpu, "silu").bfloat16().float()
+            r["parity_ok"] = bool(oracle.within_tolerance(y[rows.to(dev)], hidden @ w3_cpu.float())[0])
+            del w3, y
+        del x, w, z
 
     # C5: int8 -> int32
-    a_cpu, b_cpu = oracle.make_inputs("C5")
-    a, b = a_cpu.to(dev), b_cpu.to(dev)
-    cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
-    c = torch.empty((8192, 8192), device=dev, dtype=torch.int32)
-    l5 = mm.matmul_kernel.prepare(a, b, c, 8192, 8192, 8192, 8192, 1, 8192, 1, 8192, 1, **cfg)
-    r = measure("C5", lambda i: l5(), 1099511627776, 402653184, "i8", "mfma")
-    r["tile"] = cfg
-    rows = torch.arange(0, 8192, 1021)
-    r["bit_exact"] = bool(torch.equal(c[rows.to(dev)].cpu(), oracle.reference_matmul(a_cpu[rows], b_cpu)))
-    if not args.no_vendor and hasattr(torch, "_int_mm"):
-        try:
-            r["vendor_ms"] = vendor_ms(lambda i: torch._int_mm(a, b))
-        except Exception as e:                      # the vendor path is optional; its absence is not an error here
-            r["vendor_ms"] = None
-            r["vendor_note"] = f"torch._int_mm unavailable: {type(e).__name__}"
-    if not args.no_cpu:
-        nr = 256
-        ad, bd = a_cpu[:nr].double(), b_cpu.double()
-        t, n = cpu_time(lambda: torch.matmul(ad, bd))
-        r["cpu"] = {"ms": round(t * 1e3, 3), "gops": round(1099511627776 * nr / 8192 / t / 1e9, 1),
-                    "cores": torch.get_num_threads(),
-                    "sample": f"torch fp64 CPU matmul (exact for int8), first {nr} of 8192 rows, median of {n}"}
+    if "C5" in wanted:
+        a_cpu, b_cpu = operands("C5")
+        a, b = a_cpu.to(dev), b_cpu.to(dev)
+        cfg = pick_config(mm.matmul_kernel, lambda c: mm._launch_matmul(a, b, c), a, b, args.tune)
+        c = torch.empty((8192, 8192), device=dev, dtype=torch.int32)
+        l5 = mm.matmul_kernel.prepare(a, b, c, 8192, 8192, 8192, 8192, 1, 8192, 1, 8192, 1, **cfg)
+        r = measure("C5", lambda i: l5(), 1099511627776, 402653184, "i8", "mfma")
+        r["tile"] = cfg
+        rows = torch.arange(0, 8192, 1021)
+        r["bit_exact"] = bool(torch.equal(c[rows.to(dev)].cpu(), oracle.reference_matmul(a_cpu[rows], b_cpu)))
+        if not args.no_vendor and hasattr(torch, "_int_mm"):
+            try:
+                r["vendor_ms"] = vendor_ms(lambda i: torch._int_mm(a, b))
+            except Exception as e:                      # the vendor path is optional; its absence is not an error here
+                r["vendor_ms"] = None
+                r["vendor_note"] = f"torch._int_mm unavailable: {type(e).__name__}"
+        if not args.no_cpu:
+            nr = 256
+            ad, bd = a_cpu[:nr].double(), b_cpu.double()
+            t, n = cpu_time(lambda: torch.matmul(ad, bd))
+            r["cpu"] = {"ms": round(t * 1e3, 3), "gops": round(1099511627776 * nr / 8192 / t / 1e9, 1),
+                        "cores": torch.get_num_threads(),
+                        "sample": f"torch fp64 CPU matmul (exact for int8), first {nr} of 8192 rows, median of {n}"}
     return res
 
 

@@ -50,6 +50,28 @@ enum tnx_epilogue {
   TNX_EPI_GLU_IDENTITY = 3  /* gate * lin (the reference's fall-through branch)  */
 };
 
+/* how tiles are handed to workgroups (flags, may be combined) */
+enum tnx_schedule {
+  TNX_SCHED_DEFAULT = 0,    /* one workgroup per tile; launch order = XCD-aware remap + tl.swizzle2d(group_m),
+                               the order of tritonix/ops/matmul.py:70                                           */
+  TNX_SCHED_PERSISTENT = 1, /* one workgroup per CU walks its tiles; the next tile's first K slabs load while
+                               the current tile's epilogue runs (the reference's draft of the same idea:
+                               playground/persistent_mma.py:47-141).  Needs split_k == 1, the DMA layout,
+                               k >= num_stages * block_k and a tile built with this variant, else
+                               TNX_E_UNSUPPORTED                                                                */
+  TNX_SCHED_SUPERBLOCK = 2, /* launch order = 16x16 super-blocks of tiles walked in serpentine order, an 8x4
+                               sub-block per XCD: consecutive rounds of 256 workgroups share half of their
+                               operand panels.  Ignored (default order) when split_k > 1                       */
+  TNX_SCHED_ATOMIC_REDUCE = 4 /* split_k > 1: the K slices are added into ONE fp32 / int32 copy of each cut tile
+                               with device-scope atomic adds (the reference adds with tl.atomic_add too,
+                               tritonix/ops/matmul.py:202, but into C and after rounding to the output type;
+                               here the sum stays fp32 and is rounded once) instead of being stored apart and
+                               summed in slice order.  Float results then depend on arrival order in the
+                               last bits.  The workspace bytes [TNX_WS_COUNTER_BYTES, TNX_WS_COUNTER_BYTES +
+                               cut tiles * block_m * block_n * 4) must be zero when the launch starts; the
+                               launch leaves them zero (an ordered-mode launch on the same workspace does not) */
+};
+
 /* status codes */
 enum tnx_status {
   TNX_OK = 0,
@@ -81,7 +103,7 @@ typedef struct tnx_gemm_args {
   int32_t num_warps;  /* wavefronts (64 lanes) per workgroup: 4 or 8             */
   int32_t epilogue;   /* tnx_epilogue                                            */
   int32_t tail_tiles; /* with split_k > 1: 0 = every tile is cut; t > 0 = see below    */
-  int32_t reserved0;  /* must be 0                                               */
+  int32_t schedule;   /* tnx_schedule flags, 0 = one workgroup per tile in tl.swizzle2d order */
   void* workspace;    /* device scratch for split_k > 1 (see tnx_gemm_workspace_bytes) */
   size_t workspace_bytes;
   void* stream;       /* hipStream_t; NULL = the null stream                     */
@@ -138,8 +160,15 @@ int tnx_gemm_supported(const tnx_gemm_args* args);
  * and tail_tiles to 0. */
 int tnx_gemm_default_config(tnx_gemm_args* args);
 
+/* Which tile the workgroup with launch-order id `id` computes (no split): the host-side copy of the device
+ * functions, for tests and tooling.  Default schedule: XCD-aware remap followed by tl.swizzle2d with
+ * size_g = group_m (tritonix/ops/matmul.py:70; triton/language/standard.py:80-116).  With
+ * TNX_SCHED_SUPERBLOCK: the super-block order.  Either is a bijection of [0, tiles_m*tiles_n) onto the grid. */
+int tnx_tile_coords(int schedule, int id, int tiles_m, int tiles_n, int group_m, int* tile_m, int* tile_n);
+
 /* Number of compiled tile kernels, and a description of the i-th one:
- * "dtype bm bn bk warps stages" as a NUL-terminated string (static storage). */
+ * "dtype bm bn bk warps stages [generic] [persistent]" as a NUL-terminated string (static storage);
+ * "generic": also built with the element-wise loader; "persistent": also built for TNX_SCHED_PERSISTENT. */
 int tnx_kernel_count(void);
 const char* tnx_kernel_name(int i);
 

@@ -149,8 +149,10 @@ def test_default_config_of_the_benchmark_shapes():
     def pick(dt, out, m, n, k):
         g = args(m=m, n=n, k=k, stride_am=k, stride_bk=n, stride_cm=n, in_dtype=dt, out_dtype=out)
         lib.tnx_gemm_default_config(ctypes.byref(g))
+        picked.append(g.schedule)
         return (g.block_m, g.block_n, g.block_k, g.num_warps, g.num_stages, g.split_k, g.tail_tiles)
 
+    picked = []
     assert pick(_C.BF16, _C.BF16, 8192, 8192, 8192) == (256, 256, 64, 4, 2, 1, 0)
     assert pick(_C.BF16, _C.BF16, 4096, 28672, 4096) == (256, 256, 64, 4, 2, 1, 0)
     assert pick(_C.I8, _C.I32, 8192, 8192, 8192) == (256, 256, 128, 4, 2, 1, 0)
@@ -160,3 +162,5 @@ def test_default_config_of_the_benchmark_shapes():
     assert pick(_C.BF16, _C.BF16, 6144, 6144, 6144) == (256, 256, 64, 4, 2, 4, 64)
     # 400 tiles: 144 trailing tiles cannot be cut without spilling into another wave
     assert pick(_C.BF16, _C.BF16, 5120, 5120, 8192) == (256, 256, 64, 4, 2, 1, 0)
+    # grids of at least 16 x 16 uncut tiles are walked in super-block order; nothing is made persistent by default
+    assert picked == [_C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, 0, 0, 0, _C.SCHED_SUPERBLOCK]

@@ -30,7 +30,7 @@ def test_arguments_land_in_the_struct():
     assert (g.stride_am, g.stride_ak, g.stride_bk, g.stride_bn, g.stride_cm, g.stride_cn) == (512, 1, 384, 1, 384, 1)
     assert (g.in_dtype, g.out_dtype) == (_C.BF16, _C.BF16)
     assert (g.block_m, g.block_n, g.block_k, g.group_m, g.num_stages, g.num_warps) == (128, 128, 64, 8, 2, 4)
-    assert (g.split_k, g.tail_tiles, g.epilogue, g.reserved0) == (1, 0, _C.EPI_NONE, 0)
+    assert (g.split_k, g.tail_tiles, g.epilogue, g.schedule) == (1, 0, _C.EPI_NONE, 0)
     assert (g.a, g.b, g.c) == (a.data_ptr(), b.data_ptr(), c.data_ptr())
     assert _C.load().tnx_gemm_supported(ctypes.byref(g)) == _C.OK
 
@@ -106,7 +106,7 @@ def test_new_kernel_objects_follow_the_same_protocol():
     k = HipKernel("probe", ["block_m", "block_n", "block_k", "group_m", "num_stages", "num_warps"])
     assert k.arg_names[:12] == ["a", "b", "c", "m", "n", "k", "stride_am", "stride_ak", "stride_bk", "stride_bn",
                                 "stride_cm", "stride_cn"]
-    assert k.arg_names[-2:] == ["split_k", "tail_tiles"]
+    assert k.arg_names[-5:] == ["split_k", "tail_tiles", "persistent", "superblock", "atomic_reduce"]
     seen = []
     k.add_pre_run_hook(lambda *a, **kw: seen.append(kw.get("block_m")))
     a, b, c = tensors()

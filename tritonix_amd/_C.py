@@ -12,18 +12,22 @@ from typing import Optional
 
 from tritonix_amd.testing import LDS_LIMIT_BYTES, OutOfResources
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtritonix_hip.so")
+# TRITONIX_HIP_LIB names another build of the same library (development builds of a few tiles)
+LIB_PATH = os.environ.get("TRITONIX_HIP_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                                              "libtritonix_hip.so")
 
 # enum tnx_dtype
 F16, BF16, I8, I32, F32 = 0, 1, 2, 3, 4
 # enum tnx_epilogue
 EPI_NONE, EPI_GLU_SILU, EPI_GLU_SIGMOID, EPI_GLU_IDENTITY = 0, 1, 2, 3
+# enum tnx_schedule (flags)
+SCHED_DEFAULT, SCHED_PERSISTENT, SCHED_SUPERBLOCK, SCHED_ATOMIC_REDUCE = 0, 1, 2, 4
 # enum tnx_status
 OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP, E_STATIC_LIMIT = 0, 1, 2, 3, 4, 5, 6
 STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
-           "tnx_gemm_default_config", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
+           "tnx_gemm_default_config", "tnx_tile_coords", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
            "tnx_last_hip_error", "tnx_version")
 
 
@@ -39,7 +43,7 @@ class GemmArgs(ctypes.Structure):
         ("block_m", ctypes.c_int32), ("block_n", ctypes.c_int32), ("block_k", ctypes.c_int32),
         ("group_m", ctypes.c_int32), ("split_k", ctypes.c_int32),
         ("num_stages", ctypes.c_int32), ("num_warps", ctypes.c_int32),
-        ("epilogue", ctypes.c_int32), ("tail_tiles", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("epilogue", ctypes.c_int32), ("tail_tiles", ctypes.c_int32), ("schedule", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
     ]
@@ -70,6 +74,8 @@ def load() -> ctypes.CDLL:
     lib.tnx_gemm_supported.restype = ctypes.c_int
     lib.tnx_gemm_default_config.argtypes = [p]
     lib.tnx_gemm_default_config.restype = ctypes.c_int
+    lib.tnx_tile_coords.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_int)] * 2
+    lib.tnx_tile_coords.restype = ctypes.c_int
     lib.tnx_kernel_count.argtypes = []
     lib.tnx_kernel_count.restype = ctypes.c_int
     lib.tnx_kernel_name.argtypes = [ctypes.c_int]
@@ -104,6 +110,15 @@ def raise_for_status(status: int, args: GemmArgs) -> None:
     if status in (E_WORKSPACE, E_STATIC_LIMIT):
         raise RuntimeError(strerror(status))
     raise ValueError(strerror(status))
+
+
+def tile_coords(schedule: int, idx: int, tiles_m: int, tiles_n: int, group_m: int = 8):
+    """(tile_m, tile_n) the workgroup with launch-order id ``idx`` computes under ``schedule`` (host arithmetic)."""
+    tm, tn = ctypes.c_int(), ctypes.c_int()
+    status = load().tnx_tile_coords(schedule, idx, tiles_m, tiles_n, group_m, ctypes.byref(tm), ctypes.byref(tn))
+    if status != OK:
+        raise ValueError(strerror(status))
+    return tm.value, tn.value
 
 
 def kernel_names():

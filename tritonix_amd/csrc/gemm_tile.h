@@ -54,6 +54,8 @@ struct GemmParams {
   int out_dtype;
   bool c_vec_ok;          // C takes 16-byte stores along n (stride_cn == 1, 16-byte aligned rows)
   bool b_once;            // every element of B is read by exactly one workgroup (one tile row): stream it non-temporally
+  int tile_order;         // 0: XCD remap + tl.swizzle2d(group_m); 1: 16x16 super-blocks in serpentine order (superblock_order)
+  int atomic_reduce;      // split-K: slices are added into one fp32/int32 copy with device-scope atomics instead of being kept apart
 };
 
 // ---------------------------------------------------------------------------
@@ -125,16 +127,71 @@ __host__ __device__ inline void swizzle2d(int i, int j, int size_i, int size_j, 
   *oj = r / g;
 }
 
+// Chip-level tile order for grids much larger than the CU count.  The 256 workgroups that run
+// together (one per CU) take one 16x16 super-block of tiles, so one "round" touches 16 row panels
+// of A and 16 column panels of B; super-blocks are walked in serpentine order, so consecutive
+// rounds share half of their operands (which then come from the 256 MiB memory-side cache instead
+// of HBM); inside a super-block each XCD owns an 8x4 sub-block (12 panels through its L2).
+// A bijection from [0, tiles_m*tiles_n) onto the tile grid for every grid size.
+__host__ __device__ inline void superblock_order(int pid, int tiles_m, int tiles_n, int* pm, int* pn) {
+  constexpr int SB = 16, CHUNK = SB * SB;
+  const int total = tiles_m * tiles_n;
+  // ids congruent mod 8 (one XCD) become one run inside each aligned chunk of 256 ids
+  const int chunk0 = pid - pid % CHUNK;
+  const int csize = total - chunk0 < CHUNK ? total - chunk0 : CHUNK;
+  const int s = chunk0 + xcd_remap(pid - chunk0, csize, 8);
+  // s-th tile of the walk: rows of super-blocks top to bottom, alternating direction
+  const int row_tiles = SB * tiles_n;
+  const int i = s / row_tiles;
+  int rem = s - i * row_tiles;
+  const int h = tiles_m - i * SB < SB ? tiles_m - i * SB : SB;
+  const int nsb = (tiles_n + SB - 1) / SB;
+  const int wlast = tiles_n - (nsb - 1) * SB;
+  const bool rev = i & 1;
+  int jw, w;
+  if (!rev) {
+    jw = rem / (h * SB);
+    if (jw > nsb - 1) jw = nsb - 1;
+    w = jw == nsb - 1 ? wlast : SB;
+    rem -= jw * h * SB;
+  } else if (rem < h * wlast) {
+    jw = 0;
+    w = wlast;
+  } else {
+    rem -= h * wlast;
+    jw = 1 + rem / (h * SB);
+    w = SB;
+    rem -= (jw - 1) * h * SB;
+  }
+  const int j = rev ? nsb - 1 - jw : jw;
+  int r, c;
+  if (h == SB && w == SB) {
+    const int sub = rem / 32, idx = rem % 32;     // XCD sub-block: 2 x 4 of them, each 8 rows x 4 columns, walked down the rows
+    r = 8 * (sub / 4) + idx % 8;
+    c = 4 * (sub % 4) + idx / 8;
+  } else {
+    r = rem % h;
+    c = rem / h;
+  }
+  *pm = i * SB + r;
+  *pn = j * SB + c;
+}
+
 // vmcnt-only wait (lgkmcnt and expcnt left at "no wait") in the gfx9 encoding
 #define TNX_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | ((((n) >> 4) & 0x3) << 14) | 0x0F70)
 
 // 16 bytes per lane, global -> LDS without touching VGPRs.  LDS destination is
-// lds_base + lane*16 (lds_base wave-uniform, carried in M0).
+// lds_base + lane*16 (lds_base wave-uniform, carried in M0).  M0 is written inside the asm and
+// cannot be named as clobbered (the compiler reserves it and rejects it in a clobber list); that
+// is sound only while no compiler-generated instruction of these kernels reads M0 -- none does
+// (no register-indexed arrays, no LDS-direct or GWS operations: every array is fully unrolled).
+// The builtin form of this load is not used because the compiler then waits for vmcnt(0) before
+// every later LDS read, which serialises the ring.
 __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
-               : "memory", "m0");
+               : "memory");
 }
 
 // same, with the non-temporal hint: for an operand that is streamed from HBM once and never reused
@@ -142,7 +199,7 @@ __device__ __forceinline__ void dma16_nt(const uint8_t* sbase, uint32_t voff, ui
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                :
                : "s"(lds_base), "v"(voff), "s"(sbase)
-               : "memory", "m0");
+               : "memory");
 }
 
 __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
@@ -215,7 +272,11 @@ struct TileCfg {
   static constexpr int WGM = (NW == 4) ? 2 : (BM > BN ? 4 : 2);  // wave grid
   static constexpr int WGN = NW / WGM;
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;            // wave tile
+#ifdef TNX_EXP_MI16
+  static constexpr int MI = 16;
+#else
   static constexpr int MI = (WTM % 32 == 0 && WTN % 32 == 0) ? 32 : 16;
+#endif
   static constexpr int TM = WTM / MI, TN = WTN / MI;
   static constexpr int KB = (MI == 32) ? 32 : 64;                 // k bytes one MFMA consumes
   static constexpr int MMA_K = KB / ES;
@@ -304,6 +365,7 @@ struct SliceSrc {
   const uint8_t* base;     // this wave's part of slice 0
   uint32_t slice_stride;   // bytes from one slice to the next (the host keeps nslices * slice_stride under 4 GiB)
   int nslices;
+  bool rezero;             // atomic reduction: the one slice holds the finished sums; it is cleared again after the read
 };
 
 // Sum of the split-K slices of one row-block of a wave, group by group, into the wave's LDS
@@ -330,6 +392,11 @@ __device__ __forceinline__ void sum_slices(__amdgpu_buffer_rsrc_t win, uint32_t 
           const int z = z0 + u < src.nslices ? z0 + u : src.nslices - 1;
           w[x * ZB + u] = load16_agent(win, q0 + (uint32_t)(jg0 + x) * 1024u + (uint32_t)z * src.slice_stride);
         }
+      if (src.rezero) {
+        // atomic reduction: what was just read is the sum; leave zeros behind for the next launch
+#pragma unroll
+        for (int x = 0; x < G; ++x) store16_agent(win, q0 + (uint32_t)(jg0 + x) * 1024u, i32x4{0, 0, 0, 0});
+      }
 #pragma unroll
       for (int x = 0; x < G; ++x)
 #pragma unroll
@@ -441,6 +508,95 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
   }
 }
 
+// Epilogue of the persistent kernel.  The ring is already being refilled with the next tile's
+// first slabs while this runs, so the accumulators pass through a small strip of their own: 8 KiB
+// per wave = 32 rows x 64 accumulator columns (two 32x32 MFMA tiles side by side), rows 256 bytes
+// apart with the 16-byte chunk index XOR-ed with the row, so neither the column-wise writes nor
+// the row-wise read-back collide on banks.  FULL: the tile lies inside C and C takes 16-byte
+// stores, so the number of store instructions per wave is the compile-time STORES (the caller's
+// vmcnt arithmetic relies on it).
+template <class C> struct PairStrip {
+  static constexpr int WAVE_BYTES = 32 * 256;
+  static constexpr int BYTES = C::NW * WAVE_BYTES;
+};
+template <class T, class C, class O, bool GLU> struct PairEpilogue {
+  typedef typename T::acc_s acc_s;
+  typedef Pack16<O, acc_s, GLU> PK;
+  static constexpr int OCOLS = GLU ? 32 : 64;                 // output columns per pass
+  static constexpr int CPRW = OCOLS / PK::OUTV;               // lanes per output row
+  static constexpr int ITERS = 32 * CPRW / 64;
+  static constexpr int CH = PK::NF / 4;                       // 16-byte chunks one lane reads back
+  static constexpr int STORES = C::TM * (C::TN / 2) * ITERS;  // store instructions per wave on a FULL tile
+};
+template <class T, class C, class O, bool GLU, bool FULL, class ACC>
+__device__ __forceinline__ void epilogue_store_pairs(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t strip, int lane,
+                                                     int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
+                                                     int64_t scn, bool vec_ok, int epi) {
+  static_assert(C::MI == 32 && C::TN % 2 == 0, "pair strips need 32x32 MFMA tiles in an even number of columns");
+  typedef PairEpilogue<T, C, O, GLU> E;
+  typedef typename E::acc_s acc_s;
+  typedef typename E::PK PK;
+  typedef typename PK::raw raw;
+  typedef acc_s acc4 __attribute__((ext_vector_type(4)));
+  raw* cp = (raw*)cbase;
+  const int wrow = lane & 31, wk = lane >> 5;
+  const uint32_t wbase = strip + wrow * 256;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+    if (!FULL && gm0 + i * 32 >= m) break;
+#pragma unroll
+    for (int jp = 0; jp < C::TN / 2; ++jp) {
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int c = jj * 8 + g * 2 + wk;                  // chunk of four columns inside the 64-column pass
+          *TNX_LDS(acc4, wbase + ((c ^ (wrow & 15)) << 4)) =
+              acc4{acc[i][2 * jp + jj][4 * g + 0], acc[i][2 * jp + jj][4 * g + 1], acc[i][2 * jp + jj][4 * g + 2],
+                   acc[i][2 * jp + jj][4 * g + 3]};
+        }
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the strip is private to the wave
+      acc_s f[E::ITERS][PK::NF];
+#pragma unroll
+      for (int it = 0; it < E::ITERS; ++it) {
+        const int q = it * 64 + lane;
+        const int row = q / E::CPRW, cc = q % E::CPRW;
+#pragma unroll
+        for (int x = 0; x < E::CH; ++x) {
+          const i32x4 v = *TNX_LDS(i32x4, strip + row * 256 + (((cc * E::CH + x) ^ (row & 15)) << 4));
+          __builtin_memcpy(&f[it][4 * x], &v, 16);
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < E::ITERS; ++it) {
+        const int q = it * 64 + lane;
+        const int row = q / E::CPRW, cc = q % E::CPRW;
+        const int64_t gm = gm0 + i * 32 + row;
+        const int64_t gc = gc0 + jp * E::OCOLS + cc * PK::OUTV;
+        raw out[PK::OUTV];
+        PK::run(f[it], epi, out);
+        raw* dst = cp + gm * scm + gc * scn;
+        if (FULL) {
+          i32x4 v;
+          __builtin_memcpy(&v, out, 16);
+          *(i32x4*)dst = v;
+        } else if (gm < m) {
+          if (vec_ok && gc + PK::OUTV <= ncols) {
+            i32x4 v;
+            __builtin_memcpy(&v, out, 16);
+            *(i32x4*)dst = v;
+          } else {
+#pragma unroll 1
+            for (int x = 0; x < PK::OUTV; ++x)
+              if (gc + x < ncols) dst[x * scn] = out[x];
+          }
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // the next pass overwrites the strip
+    }
+  }
+}
+
 // The first WS_COUNTER_BYTES of the split-K workspace hold one arrival counter per cut tile.
 // They must be zero when a launch starts; every launch leaves them zero.
 constexpr int WS_COUNTER_BYTES = 65536;
@@ -454,7 +610,7 @@ constexpr int WS_MAX_TILES = WS_COUNTER_BYTES / 4;
 // L2s) are avoided on purpose: they cost more than the GEMM.
 template <class T, class C, class ACC>
 __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t* wave_slice, uint32_t lds_strip, int lane,
-                                              int64_t gm0, int64_t m, int* counter, int* flag, int nslices) {
+                                              int64_t gm0, int64_t m, int* counter, int* flag, int nslices, bool atomic) {
   typedef typename T::acc_s acc_s;
   typedef acc_s acc4 __attribute__((ext_vector_type(4)));
   constexpr int NGRP = C::ACC_N / 4;
@@ -463,6 +619,21 @@ __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t*
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
     if (gm0 + i * C::MI >= m) break;
+    if (atomic) {
+      // every slice adds into the same copy (wave_slice is slice 0 for all of them); same element order as a stored slice
+      if (gm0 + i * C::MI + lane % C::MI < m) {
+        acc_s* dst = (acc_s*)(wave_slice + (int64_t)i * NQ * 1024 + lane * 16);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+          for (int g = 0; g < NGRP; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              __hip_atomic_fetch_add(dst + (j * NGRP + g) * 256 + e, acc[i][j][4 * g + e], __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+      }
+      continue;
+    }
     // registers -> LDS -> registers keeps the copy loop rolled (the accumulators may sit in AGPRs,
     // which a 16-byte device-scope store cannot name directly)
 #pragma unroll
@@ -501,16 +672,21 @@ template <bool B> struct BoolTag { static constexpr bool value = B; };
 // ---------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------
-template <class T, class C, bool FAST>
+template <class T, class C, bool FAST, bool PERSIST = false>
 __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
   constexpr int MI = C::MI, TM = C::TM, TN = C::TN;
   static_assert(C::VALID, "tile configuration not supported by this kernel");
+  static_assert(!PERSIST || FAST, "the persistent kernel is built with the DMA loader only");
   typedef Mma<T, MI> MMA;
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
 
-  constexpr int SMEM_BYTES = C::LDS_BYTES > EpiStage<C>::BYTES ? C::LDS_BYTES : EpiStage<C>::BYTES;
+  // one workgroup per tile: the epilogue strips are laid over the ring once the K loop is done.
+  // persistent: the ring is refilled for the next tile during the epilogue, so the strips follow it.
+  constexpr int RING_OR_STRIPS = C::LDS_BYTES > EpiStage<C>::BYTES ? C::LDS_BYTES : EpiStage<C>::BYTES;
+  constexpr int SMEM_BYTES = PERSIST ? C::LDS_BYTES + PairStrip<C>::BYTES : RING_OR_STRIPS;
+  static_assert(SMEM_BYTES <= 163840, "LDS budget of one CU exceeded");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[SMEM_BYTES];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
 
@@ -522,60 +698,80 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // Tiles [0, split_tile0) in launch order are computed whole by one workgroup each; the
   // tiles after them are cut split_k ways along K (all tiles when split_tile0 == 0: plain
   // split-K; only the last partial wave of tiles when the tile count does not fill the CUs).
+  // The persistent kernel never cuts: workgroup b computes tiles b, b + gridDim.x, ... whole.
   const int ntiles = p.tiles_m * p.tiles_n;
-  int split = 0, logical;
+  int split = 0, logical = 0;
   bool cut = false;
-  if ((int)blockIdx.x < p.split_tile0) {
-    logical = xcd_remap(blockIdx.x, p.split_tile0, 8);
-  } else {
-    const int ncut = ntiles - p.split_tile0;
-    int t = blockIdx.x - p.split_tile0;
-    split = t / ncut;
-    t -= split * ncut;
-    logical = p.split_tile0 + xcd_remap(t, ncut, 8);
-    cut = p.split_k > 1;
-  }
+  // launch-order id -> tile coordinates
+  auto locate = [&](int id, int* pid_m, int* pid_n) {
+    if (p.tile_order == 1) {
+      superblock_order(id, p.tiles_m, p.tiles_n, pid_m, pid_n);
+    } else {
+      const int lg = xcd_remap(id, ntiles, 8);
+      swizzle2d(lg / p.tiles_n, lg % p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, pid_m, pid_n);
+    }
+  };
   int pid_m, pid_n;
-  swizzle2d(logical / p.tiles_n, logical % p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, &pid_m, &pid_n);
-  const int64_t m0 = (int64_t)pid_m * BM, n0 = (int64_t)pid_n * BN;
+  if (PERSIST || p.split_k <= 1) {
+    locate(blockIdx.x, &pid_m, &pid_n);
+  } else {
+    if ((int)blockIdx.x < p.split_tile0) {
+      logical = xcd_remap(blockIdx.x, p.split_tile0, 8);
+    } else {
+      const int ncut = ntiles - p.split_tile0;
+      int t = blockIdx.x - p.split_tile0;
+      split = t / ncut;
+      t -= split * ncut;
+      logical = p.split_tile0 + xcd_remap(t, ncut, 8);
+      cut = true;
+    }
+    swizzle2d(logical / p.tiles_n, logical % p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, &pid_m, &pid_n);
+  }
 
   const int kt_total = (int)((p.k + BK - 1) / BK);
   const int kt0 = cut ? split * p.ktiles_per_split : 0;
   int kt1 = cut ? kt0 + p.ktiles_per_split : kt_total;
   if (kt1 > kt_total) kt1 = kt_total;
-  const int KT = kt1 > kt0 ? kt1 - kt0 : 0;          // slabs of this workgroup
+  const int KT = kt1 > kt0 ? kt1 - kt0 : 0;          // slabs of this workgroup (per tile)
   // FAST kernels are only launched when k % BK == 0 and A, B are row-major
   // and 16-byte aligned: every slab goes through the DMA path.  Otherwise every
   // slab goes through the element-wise loader.
-  const int kt_dma = FAST ? KT : 0;
 
-  // ---- DMA addressing (FAST): per-lane byte offsets, constant over the K loop
+  // ---- the tile the loader works on: origin, DMA bases and per-lane byte offsets.
+  // (In the persistent kernel the loader moves on to the next tile before the epilogue of the
+  // current one has run, so the epilogue keeps its own copy of the origin.)
+  int64_t m0 = 0, n0 = 0;
   uint32_t a_voff[C::A_LPW], b_voff[C::B_LPW];
   const uint8_t* a_sbase = p.a;
   const uint8_t* b_sbase = p.b;
-  if (FAST) {
-    const int64_t lda = p.sam, ldb = p.sbk;
-    // wave-uniform by construction; say so, so both stay in SGPRs for the DMA's scalar base operand
-    a_sbase = uniform_ptr(p.a + (m0 * lda + (int64_t)kt0 * BK) * ES);
-    b_sbase = uniform_ptr(p.b + ((int64_t)kt0 * BK * ldb + n0) * ES);
-    const int64_t mrem = p.m - 1 - m0;  // last valid row inside this tile
+  auto place_tile = [&](int tile_m, int tile_n) {
+    m0 = (int64_t)tile_m * BM;
+    n0 = (int64_t)tile_n * BN;
+    if (FAST) {
+      const int64_t lda = p.sam, ldb = p.sbk;
+      // wave-uniform by construction; say so, so both stay in SGPRs for the DMA's scalar base operand
+      a_sbase = uniform_ptr(p.a + (m0 * lda + (int64_t)kt0 * BK) * ES);
+      b_sbase = uniform_ptr(p.b + ((int64_t)kt0 * BK * ldb + n0) * ES);
+      const int64_t mrem = p.m - 1 - m0;  // last valid row inside this tile
 #pragma unroll
-    for (int q = 0; q < C::A_LPW; ++q) {
-      int P = (q * NW + wave) * 64 + lane;
-      int row = P / C::CPR_A, cs = P % C::CPR_A;
-      int c = cs ^ C::swzA(row);
-      int64_t r = row < mrem ? row : mrem;
-      a_voff[q] = (uint32_t)(r * lda * ES + c * 16);
-    }
+      for (int q = 0; q < C::A_LPW; ++q) {
+        int P = (q * NW + wave) * 64 + lane;
+        int row = P / C::CPR_A, cs = P % C::CPR_A;
+        int c = cs ^ C::swzA(row);
+        int64_t r = row < mrem ? row : mrem;
+        a_voff[q] = (uint32_t)(r * lda * ES + c * 16);
+      }
 #pragma unroll
-    for (int q = 0; q < C::B_LPW; ++q) {
-      int P = (q * NW + wave) * 64 + lane;
-      int row = P / C::CPR_B, cs = P % C::CPR_B;
-      int c = cs ^ C::swzB(row);
-      if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
-      b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
+      for (int q = 0; q < C::B_LPW; ++q) {
+        int P = (q * NW + wave) * 64 + lane;
+        int row = P / C::CPR_B, cs = P % C::CPR_B;
+        int c = cs ^ C::swzB(row);
+        if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
+        b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
+      }
     }
-  }
+  };
+  place_tile(pid_m, pid_n);
 
   // element-wise loader: any strides, any ragged edge, zero fill.  Used for
   // the K-tail slab of FAST kernels and for every slab otherwise.
@@ -676,6 +872,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   };
   auto mma_one = [&](int set, int idx) {
     int i = idx / TN, j = idx % TN;
+#ifdef TNX_EXP_SERP
+    if (i & 1) j = TN - 1 - j;
+#endif
     i32x4 b4 = i32x4{fb[set][j][0].x, fb[set][j][0].y, fb[set][j][1].x, fb[set][j][1].y};
     acc[i][j] = MMA::run(b4, fa[set][i], acc[i][j]);   // rows = n, cols = m: the tile comes out transposed
   };
@@ -755,7 +954,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   typedef BoolTag<true> Yes;
   typedef BoolTag<false> No;
 
-  if (KT > 0) {
+  // first STAGES slabs of the tile the loader stands on
+  auto issue_prologue = [&]() {
 #pragma unroll
     for (int s = 0; s < STAGES; ++s) {
       if (s < KT) {
@@ -768,7 +968,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         }
       }
     }
-    if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
+  };
+  // the K loop of one tile, from "slab 0 has landed" to the last MFMA; the prologue has been issued
+  auto k_loop = [&]() {
+  if (KT > 0) {
     __syncthreads();
     const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
 #pragma unroll
@@ -826,35 +1029,94 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
 #pragma unroll
     for (int x = 0; x < NMMA; ++x) mma_one(LAST, x);
   }
+  };
 
-  // ---- epilogue ------------------------------------------------------------
-  // every wave is done with the slabs before the LDS is reused for the output strips
-  __syncthreads();
-  const int64_t gm0 = m0 + wy * C::WTM;
-  const int64_t gn0 = n0 + wx * C::WTN;
-  const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
   typedef typename OutOf<T>::type O;
-  if (cut) {
-    // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
-    const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;
-    const int64_t slice_stride = (int64_t)ncut * BM * BN * 4;
-    uint8_t* wave0 = p.ws + WS_COUNTER_BYTES + ((int64_t)ctile * NW + wave) * (C::WTM * C::WTN * 4);
-    if (!splitk_arrive<T, C>(acc, wave0 + split * slice_stride, strip, lane, gm0, p.m, (int*)p.ws + ctile, (int*)smem,
-                             p.split_k))
-      return;
-    const SliceSrc src = {wave0, (uint32_t)slice_stride, p.split_k};
-    if (p.epilogue == EPI_NONE)
-      epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
-    else
-      epilogue_store<T, C, O, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                          p.c_vec_ok, p.epilogue);
+  if constexpr (!PERSIST) {
+    if (KT > 0) {
+      issue_prologue();
+      if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
+    }
+    k_loop();
+
+    // ---- epilogue ------------------------------------------------------------
+    // every wave is done with the slabs before the LDS is reused for the output strips
+    __syncthreads();
+    const int64_t gm0 = m0 + wy * C::WTM;
+    const int64_t gn0 = n0 + wx * C::WTN;
+    const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
+    if (cut) {
+      // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
+      const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;
+      const int64_t slice_stride = (int64_t)ncut * BM * BN * 4;
+      uint8_t* wave0 = p.ws + WS_COUNTER_BYTES + ((int64_t)ctile * NW + wave) * (C::WTM * C::WTN * 4);
+      const bool atomic = p.atomic_reduce != 0;
+      if (!splitk_arrive<T, C>(acc, wave0 + (atomic ? 0 : split * slice_stride), strip, lane, gm0, p.m, (int*)p.ws + ctile,
+                               (int*)smem, p.split_k, atomic))
+        return;
+      const SliceSrc src = {wave0, (uint32_t)slice_stride, atomic ? 1 : p.split_k, atomic};
+      if (p.epilogue == EPI_NONE)
+        epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+      else
+        epilogue_store<T, C, O, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                            p.c_vec_ok, p.epilogue);
+    } else {
+      const SliceSrc none = {nullptr, 0, 0, false};
+      if (p.epilogue == EPI_NONE)
+        epilogue_store<T, C, O, false, false>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+      else
+        epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                             p.c_vec_ok, p.epilogue);
+    }
   } else {
-    const SliceSrc none = {nullptr, 0, 0};
-    if (p.epilogue == EPI_NONE)
-      epilogue_store<T, C, O, false, false>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
-    else
-      epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                           p.c_vec_ok, p.epilogue);
+    // ---- persistent: this workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... ------------
+    // The host launches it only with KT >= STAGES.  While the epilogue of a tile runs, the first
+    // STAGES slabs of the next tile are already on their way into the ring, and the epilogue's
+    // stores drain under the next tile's first K slabs.  vmcnt retires in issue order, so
+    // "at most X operations outstanding" means the X youngest: after an epilogue these are its
+    // stores, and everything older -- the next tile's prologue -- has landed.  X may therefore
+    // include the stores only when their number is known exactly (a tile fully inside C with
+    // 16-byte stores); otherwise it is the (STAGES - 1) slabs of the prologue that may stay in
+    // flight, as for the first tile.
+    const uint32_t strip = lds0 + C::LDS_BYTES + wave * PairStrip<C>::WAVE_BYTES;
+    constexpr int X_FIRST = (STAGES - 1) * C::LPW;
+    constexpr int NST_PLAIN = PairEpilogue<T, C, O, false>::STORES, NST_GLU = PairEpilogue<T, C, O, true>::STORES;
+    constexpr int X_PLAIN = X_FIRST + NST_PLAIN > 63 ? 63 : X_FIRST + NST_PLAIN;
+    constexpr int X_GLU = X_FIRST + NST_GLU > 63 ? 63 : X_FIRST + NST_GLU;
+    const bool glu = p.epilogue != EPI_NONE;
+    issue_prologue();
+    TNX_WAIT_VM(X_FIRST);
+    for (int id = blockIdx.x; id < ntiles; id += gridDim.x) {
+      k_loop();
+      // every wave is done with the ring: it can take the next tile's first slabs
+      __syncthreads();
+      const int64_t gm0 = m0 + wy * C::WTM;
+      const int64_t gn0 = n0 + wx * C::WTN;
+      const bool full = p.c_vec_ok && m0 + BM <= p.m && n0 + BN <= p.n;
+      const int next = id + gridDim.x;
+      if (next < ntiles) {
+        int nm, nn;
+        locate(next, &nm, &nn);
+        place_tile(nm, nn);
+        issue_prologue();
+      }
+      if (!glu) {
+        if (full) epilogue_store_pairs<T, C, O, false, true>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, true, 0);
+        else epilogue_store_pairs<T, C, O, false, false>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+      } else {
+        if (full) epilogue_store_pairs<T, C, O, true, true>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, true, p.epilogue);
+        else epilogue_store_pairs<T, C, O, true, false>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{};
+      if (next < ntiles) {
+        if (!full) { TNX_WAIT_VM(X_FIRST); }
+        else if (glu) { TNX_WAIT_VM(X_GLU); }
+        else { TNX_WAIT_VM(X_PLAIN); }
+      }
+    }
   }
 }
 

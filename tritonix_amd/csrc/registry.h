@@ -14,6 +14,7 @@ struct KernelEntry {
   int lds_bytes;
   launch_fn fast;     // DMA loader: row-major, 16-byte aligned, k % bk == 0
   launch_fn generic;  // element-wise loader: any strides / ragged k; may be null
+  launch_fn persist;  // DMA loader, one workgroup per CU walking its tiles; may be null
 };
 
 struct KernelGroup {
@@ -21,12 +22,25 @@ struct KernelGroup {
   int count;
 };
 
-template <class T, class C, bool FAST>
+template <class T, class C, bool FAST, bool PERSIST = false>
 hipError_t launch_tile(const GemmParams& p, unsigned grid, hipStream_t stream) {
   static_assert(C::VALID, "tile configuration is not buildable");
-  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST>), dim3(grid), dim3(C::THREADS), 0, stream, p);
+  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST, PERSIST>), dim3(grid), dim3(C::THREADS), 0, stream, p);
   return hipGetLastError();
 }
+
+// The persistent variant exists for the large four-wave tiles whose ring leaves room for the
+// epilogue's own strips (8 KiB per wave) inside the 160 KiB of one CU.
+template <class C> constexpr bool persist_ok() {
+  return C::NW == 4 && C::BM >= 128 && C::BN >= 128 && C::MI == 32 && C::TN % 2 == 0 &&
+         C::LDS_BYTES + PairStrip<C>::BYTES <= 163840;
+}
+template <class T, class C, bool OK = persist_ok<C>()> struct PersistLaunch {
+  static constexpr launch_fn fn = nullptr;
+};
+template <class T, class C> struct PersistLaunch<T, C, true> {
+  static constexpr launch_fn fn = &launch_tile<T, C, true, true>;
+};
 
 // skinny kernel (gemm_skinny.h): tile 16 x 32 x 32, eight waves, split_k == 8 inside the workgroup,
 // num_stages = ring depth per wave.  Null when that depth / dtype is not built.
@@ -37,6 +51,7 @@ constexpr int SKINNY_STEP_BYTES = 3072;
 #define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
   {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
    &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \
-   GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr}
+   GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr,               \
+   PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
 
 }  // namespace tnx

@@ -12,7 +12,8 @@ derives its own 1-D grid from the shape and the tile.
 from __future__ import annotations
 
 import ctypes
-from typing import Callable, Dict, List, Optional, Tuple
+from collections import OrderedDict
+from typing import Callable, List, Optional, Tuple
 
 from tritonix_amd import _C
 
@@ -27,7 +28,9 @@ _POSITIONAL = ("a", "b", "c", "m", "n", "k", "stride_am", "stride_ak", "stride_b
                "stride_cn")
 _ACTIVATIONS = {"silu": _C.EPI_GLU_SILU, "sigmoid": _C.EPI_GLU_SIGMOID}
 
-_workspaces: Dict[Tuple[int, int], object] = {}
+# split-K scratch buffers, most recently used last; at most _MAX_WORKSPACES are kept alive
+_workspaces: "OrderedDict[Tuple[int, int], object]" = OrderedDict()
+_MAX_WORKSPACES = 8
 
 
 def _torch_dtype_code(dtype) -> int:
@@ -47,19 +50,38 @@ def out_dtype_for(dtype):
     return torch.int32 if dtype == torch.int8 else dtype
 
 
-def _workspace(device, stream_ptr: int, nbytes: int):
-    """Split-K scratch, one growing buffer per (device, stream).
+def _workspace_key(device, stream_ptr: int, atomic: bool = False) -> Tuple[int, int, bool]:
+    import torch
 
-    Allocated zero-filled: the leading counter region must start at zero and every launch leaves it zero.
+    return (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr, bool(atomic))
+
+
+def _workspace(device, stream_ptr: int, nbytes: int, atomic: bool = False):
+    """Split-K scratch, one growing buffer per (device, stream), the least recently used ones released.
+
+    Allocated zero-filled: the leading counter region must start at zero and every launch leaves it zero.  A
+    launch that fails part-way may leave counters set, so ``drop_workspace`` forgets the buffer after any error
+    and the next launch starts from a freshly zeroed one.
     """
     import torch
 
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    # launches that reduce with atomics need their sum region zero and leave it zero; ordered launches leave
+    # slices behind: the two modes never share a buffer
+    key = _workspace_key(device, stream_ptr, atomic)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
+    _workspaces.move_to_end(key)
+    while len(_workspaces) > _MAX_WORKSPACES:
+        _workspaces.popitem(last=False)       # launches already enqueued keep their buffer alive through the allocator's stream ordering
     return buf
+
+
+def drop_workspace(device, stream_ptr: int) -> None:
+    """Forget the scratch of (device, stream): called when a launch on it reported an error."""
+    for atomic in (False, True):
+        _workspaces.pop(_workspace_key(device, stream_ptr, atomic), None)
 
 
 class _BoundLaunch:
@@ -78,9 +100,12 @@ class HipKernel:
         self.__doc__ = doc
         self.tile_params = list(tile_params)
         self.glu = glu
-        # optional keywords after the reference's own: a K split for kernels whose signature has none, and
-        # the number of trailing tiles the split applies to (0 = all)
-        self.optional = [n for n in ("split_k", "tail_tiles") if n not in self.tile_params]
+        # optional keywords after the reference's own: a K split for kernels whose signature has none, the
+        # number of trailing tiles the split applies to (0 = all), and the two scheduling switches of the engine
+        # (persistent: one workgroup per CU walks its tiles; superblock: 16x16 super-block launch order)
+        # atomic_reduce: split-K slices are added into one fp32 copy with atomics instead of being summed in order
+        self.optional = [n for n in ("split_k", "tail_tiles", "persistent", "superblock", "atomic_reduce")
+                         if n not in self.tile_params]
         self.arg_names = (list(_POSITIONAL) + self.tile_params + (["use_tf32", "activation"] if glu else [])
                           + self.optional)
         self.pre_run_hooks: List[Callable] = []
@@ -126,6 +151,9 @@ class HipKernel:
         g.group_m = int(bound["group_m"])
         g.split_k = int(bound.get("split_k", 1))
         g.tail_tiles = int(bound.get("tail_tiles", 0))
+        g.schedule = ((_C.SCHED_PERSISTENT if int(bound.get("persistent", 0)) else 0)
+                      | (_C.SCHED_SUPERBLOCK if int(bound.get("superblock", 0)) else 0)
+                      | (_C.SCHED_ATOMIC_REDUCE if int(bound.get("atomic_reduce", 0)) else 0))
         g.num_stages, g.num_warps = int(bound["num_stages"]), int(bound["num_warps"])
         if self.glu:
             # "silu" and "sigmoid" gate explicitly; like the reference kernel, any other
@@ -170,9 +198,12 @@ class HipKernel:
         if g.split_k > 1:
             need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
             if need:
-                ws = _workspace(device, stream, need)
+                ws = _workspace(device, stream, need, bool(g.schedule & _C.SCHED_ATOMIC_REDUCE))
                 g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
-        return lib.tnx_gemm(ctypes.byref(g))
+        status = lib.tnx_gemm(ctypes.byref(g))
+        if status == _C.E_HIP and g.split_k > 1:
+            drop_workspace(device, stream)
+        return status
 
     def prepare(self, *args, **kwargs) -> Callable[[], None]:
         """Bind a launch once and return a zero-argument callable that repeats it.
@@ -191,7 +222,7 @@ class HipKernel:
         keep = [bound["a"], bound["b"], bound["c"]]
         if g.split_k > 1:
             need = int(lib.tnx_gemm_workspace_bytes(ctypes.byref(g)))
-            ws = _workspace(device, stream, need)
+            ws = _workspace(device, stream, need, bool(g.schedule & _C.SCHED_ATOMIC_REDUCE))
             g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
             keep.append(ws)
         status = lib.tnx_gemm_supported(ctypes.byref(g))
@@ -201,16 +232,20 @@ class HipKernel:
         def launch(_keep=keep, _g=g):
             st = fn(ref)
             if st:
+                if _g.split_k > 1:
+                    drop_workspace(device, stream)
                 _C.raise_for_status(st, _g)
 
         return launch
 
     # host-only helpers -------------------------------------------------
-    def lds_bytes(self, in_dtype_code: int, block_m: int, block_n: int, block_k: int, num_stages: int) -> int:
+    def lds_bytes(self, in_dtype_code: int, block_m: int, block_n: int, block_k: int, num_stages: int,
+                  num_warps: int = 4, persistent: int = 0) -> int:
         """LDS bytes per workgroup of a tile config (no GPU needed)."""
         g = _C.GemmArgs()
         g.in_dtype = in_dtype_code
-        g.block_m, g.block_n, g.block_k, g.num_stages = block_m, block_n, block_k, num_stages
+        g.block_m, g.block_n, g.block_k, g.num_stages, g.num_warps = block_m, block_n, block_k, num_stages, num_warps
+        g.schedule = _C.SCHED_PERSISTENT if persistent else 0
         return int(_C.load().tnx_gemm_lds_bytes(ctypes.byref(g)))
 
     def __repr__(self):

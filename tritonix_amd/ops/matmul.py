@@ -243,6 +243,10 @@ def default_config(a, b, split=False):
         cfg["split_k"] = g.split_k
     if g.tail_tiles > 0:
         cfg["tail_tiles"] = g.tail_tiles
+    if g.schedule & _C.SCHED_SUPERBLOCK:
+        cfg["superblock"] = 1
+    if g.schedule & _C.SCHED_PERSISTENT:
+        cfg["persistent"] = 1
     return cfg
 
 
