@@ -32,7 +32,7 @@ def test_matmul_correctness(device, M, N, K):
     assert close(torch.matmul(a, b), out), f"max diff: {(torch.matmul(a, b) - out).abs().max()}"
     ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
     assert ok and rel <= 1e-2
-    assert (M, N, K, torch.float16, True) in mm._matmul_cfg
+    assert (M, N, K, torch.float16, 1) in mm._matmul_cfg
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 512, 512), (2048, 2048, 2048)])
@@ -84,7 +84,7 @@ def test_matmul_splitk(device):
     out = tritonix_amd.matmul_splitk(a.to(device), b.to(device))
     ok, _, rel = oracle.within_tolerance(out, oracle.reference_matmul(a, b))
     assert ok and rel <= 1e-2
-    assert mm._splitk_cfg[(16, 2048, 7168, 4, torch.bfloat16, True)]["split_k"] >= 2
+    assert mm._splitk_cfg[(16, 2048, 7168, 4, torch.bfloat16, 1)]["split_k"] >= 2
 
 
 def test_glu_and_swiglu_wrappers(device):
@@ -189,8 +189,8 @@ def test_tuned_config_is_reused_from_disk(device, tmp_path, monkeypatch):
     b = torch.randn(256, 512, device=device, dtype=torch.float16)
     mm._matmul_cfg.clear()
     out1 = tritonix_amd.triton_matmul(a, b)
-    picked = mm._matmul_cfg[(384, 512, 256, torch.float16, True)]
-    assert mm.load_tuned("matmul", (384, 512, 256, torch.float16, True)) == picked
+    picked = mm._matmul_cfg[(384, 512, 256, torch.float16, 1)]
+    assert mm.load_tuned("matmul", (384, 512, 256, torch.float16, 1)) == picked
     mm._matmul_cfg.clear()
     monkeypatch.setattr(mm.matmul_kernel, "tune", lambda *a, **k: pytest.fail("tuned again despite the disk record"))
     assert torch.equal(tritonix_amd.triton_matmul(a, b), out1)
@@ -213,17 +213,19 @@ def test_memoised_config_follows_the_operand_layout(device, monkeypatch):
     for out in (out1, out2, out3):
         assert oracle.within_tolerance(out, ref)[0]
     assert torch.equal(out1, out3)
-    assert mm._matmul_cfg[(512, 384, 256, torch.float16, True)] != mm._matmul_cfg[(512, 384, 256, torch.float16, False)]
+    # row-major B (class 1) and k-contiguous B (class 2) are remembered apart
+    assert (512, 384, 256, torch.float16, 1) in mm._matmul_cfg and (512, 384, 256, torch.float16, 2) in mm._matmul_cfg
     # a misaligned base pointer is the second layout class too
     flat = torch.zeros(512 * 256 + 8, dtype=torch.float16, device=device)
     a_off = flat[1:1 + 512 * 256].view(512, 256)
     a_off.copy_(ad)
-    assert not mm.dma_layout(a_off, b_contig)
+    assert mm.dma_layout(a_off, b_contig) == 0 and mm.dma_layout(ad, b_contig) == 1 and mm.dma_layout(ad, wd.t()) == 2
     assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_off, b_contig), ref)[0]
     # a memo entry the engine refuses for these operands is replaced, not raised
-    mm._matmul_cfg[(512, 384, 256, torch.float16, False)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, True)],
-                                                                 block_m=256, block_n=256, num_stages=2, num_warps=4)
-    assert oracle.within_tolerance(tritonix_amd.triton_matmul(ad, wd.t()), ref)[0]
+    mm._matmul_cfg[(512, 384, 256, torch.float16, 0)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, 1)],
+                                                             block_m=256, block_n=256, num_stages=2, num_warps=4)
+    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_off, b_contig), ref)[0]
+    assert mm._matmul_cfg[(512, 384, 256, torch.float16, 0)]["block_m"] == 128       # replaced by the built-in choice
     mm._matmul_cfg.clear()
 
 

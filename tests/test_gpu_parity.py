@@ -311,3 +311,38 @@ def test_skinny_wave_split_kernel(device, m, n, k, stages, dtype):
         with pytest.raises(ValueError):  # and it only takes up to sixteen rows
             big = torch.zeros(17, k, dtype=dtype, device=device)
             gemm(big, b.to(device), config, kernel=gemm_splitk_kernel)
+
+
+# ---- k-contiguous B: the layout of x @ w.t() with a row-major weight ---------------------------
+@pytest.mark.parametrize("dtype,tile,shape", [
+    (torch.bfloat16, (256, 256, 64, 4, 2), (1024, 1024, 512)),
+    (torch.bfloat16, (256, 256, 64, 4, 2), (1000, 1303, 512)),     # ragged rows and an odd number of columns
+    (torch.bfloat16, (128, 128, 64, 4, 3), (300, 264, 192)),
+    (torch.float16, (64, 64, 64, 4, 4), (1024, 768, 512)),
+    (torch.int8, (256, 256, 128, 4, 2), (1024, 1000, 1024)),
+    (torch.int8, (64, 128, 128, 4, 3), (64, 2051, 2048)),
+    (torch.bfloat16, (64, 128, 64, 8, 3), (16, 4096, 14336)),      # the skinny benchmark shape against w.t(), K cut 8 ways
+], ids=lambda v: str(v).replace("torch.", "").replace(" ", ""))
+def test_k_contiguous_b_takes_its_own_dma_loader(device, dtype, tile, shape):
+    m, n, k = shape
+    g = torch.Generator("cpu").manual_seed(m + n + k)
+    if dtype == torch.int8:
+        a = torch.randint(-127, 128, (m, k), generator=g, dtype=dtype)
+        w = torch.randint(-127, 128, (n, k), generator=g, dtype=dtype)
+    else:
+        a = torch.randn(m, k, generator=g).to(dtype)
+        w = (torch.randn(n, k, generator=g) / k ** 0.5).to(dtype)
+    ad, wd = a.to(device), w.to(device)
+    b = wd.t()
+    assert b.stride() == (1, k)
+    extra = dict(split_k=8) if m == 16 else {}
+    kernel = gemm_splitk_kernel if extra else matmul_kernel
+    out = gemm(ad, b, cfg(*tile, **extra), kernel=kernel)
+    ref = oracle.reference_matmul(a, w.t())
+    if dtype == torch.int8:
+        assert torch.equal(out.cpu(), ref)
+    else:
+        check_fp(out, ref)
+        if n % 8 == 0:
+            # the same K order as the row-major loader on a contiguous copy: the same bits
+            assert torch.equal(out, gemm(ad, b.contiguous(), cfg(*tile, **extra), kernel=kernel))

@@ -63,15 +63,17 @@ def test_persistent_needs_a_built_variant_and_no_split():
     def status(**kw):
         g = _C.GemmArgs()
         base = dict(m=1024, n=1024, k=1024, stride_am=1024, stride_ak=1, stride_bk=1024, stride_bn=1, stride_cm=1024,
-                    stride_cn=1, in_dtype=_C.BF16, out_dtype=_C.BF16, block_m=256, block_n=256, block_k=64, group_m=8,
+                    stride_cn=1, in_dtype=_C.BF16, out_dtype=_C.BF16, block_m=256, block_n=128, block_k=64, group_m=8,
                     split_k=1, num_stages=2, num_warps=4, epilogue=_C.EPI_NONE, schedule=_C.SCHED_PERSISTENT)
         base.update(kw)
         for k, v in base.items():
             setattr(g, k, v)
         return lib.tnx_gemm_supported(ctypes.byref(g)), lib.tnx_gemm_lds_bytes(ctypes.byref(g))
 
-    assert status() == (_C.OK, 131072 + 4 * 8192)                         # ring + the epilogue's own strips
-    assert status(schedule=0)[1] == 131072
+    ring = 2 * (256 * 64 + 64 * 128) * 2
+    assert status() == (_C.OK, ring + 4 * 16 * 256)                           # ring + the epilogue's own strips
+    assert status(schedule=0)[1] == ring
+    assert status(block_n=256)[0] == _C.E_UNSUPPORTED                     # 256x256: its accumulators leave no registers for the tile loop
     assert status(split_k=2)[0] == _C.E_UNSUPPORTED                       # persistent tiles are never cut
     assert status(k=64)[0] == _C.E_UNSUPPORTED                            # fewer K slabs than ring stages
     assert status(block_m=64, block_n=64, num_stages=4)[0] == _C.E_UNSUPPORTED   # small tiles have no persistent variant
@@ -104,8 +106,8 @@ SCHEDULES = [dict(persistent=1), dict(superblock=1), dict(persistent=1, superblo
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,tile", [(torch.bfloat16, (256, 256, 64, 4, 2)), (torch.float16, (128, 128, 64, 4, 3)),
-                                        (torch.bfloat16, (256, 128, 64, 4, 2)), (torch.int8, (256, 256, 128, 4, 2)),
+@pytest.mark.parametrize("dtype,tile", [(torch.bfloat16, (128, 256, 64, 4, 2)), (torch.float16, (128, 128, 64, 4, 3)),
+                                        (torch.bfloat16, (256, 128, 64, 4, 2)), (torch.int8, (256, 128, 128, 4, 2)),
                                         (torch.int8, (128, 128, 128, 4, 2))],
                          ids=lambda v: str(v).replace("torch.", ""))
 @pytest.mark.parametrize("shape", [(2304, 2560, 1024), (1000, 4624, 512), (256, 256, 256), (4352, 4352, 256)],
@@ -135,12 +137,12 @@ def test_every_schedule_gives_the_bits_of_the_default_schedule(device, dtype, ti
 @pytest.mark.gpu
 @pytest.mark.parametrize("activation", ["silu", "sigmoid", "identity"])
 def test_persistent_glu_epilogue(device, activation):
-    x, w12 = oracle.make_inputs("C4", scale_down=4)          # x[1024,1024], w12[1024,7168]: 4 x 28 tiles of 256
+    x, w12 = oracle.make_inputs("C4", scale_down=4)          # x[1024,1024], w12[1024,7168]: 4 x 56 tiles of 256x128
     xd, wd = x.to(device), w12.to(device)
     outs = []
     for extra in [dict()] + SCHEDULES:
         z = torch.full((x.shape[0], w12.shape[1] // 2), 7, device=device, dtype=torch.bfloat16)
-        launch(glu_kernel, xd, wd, z, cfg(256, 256, 64, 4, 2, **extra), activation=activation)
+        launch(glu_kernel, xd, wd, z, cfg(256, 128, 64, 4, 2, **extra), activation=activation)
         outs.append(z)
     assert oracle.within_tolerance(outs[0], oracle.reference_glu(x, w12, activation))[0]
     for z in outs[1:]:
@@ -148,10 +150,10 @@ def test_persistent_glu_epilogue(device, activation):
     # a ragged problem: rows and gated columns that end inside a tile, output with a row pitch
     xr, wr = xd[:900], wd[:, :2 * 1300].contiguous()
     base = torch.full((900, 1300), 7, device=device, dtype=torch.bfloat16)
-    launch(glu_kernel, xr, wr, base, cfg(256, 256, 64, 4, 2), activation=activation)
+    launch(glu_kernel, xr, wr, base, cfg(256, 128, 64, 4, 2), activation=activation)
     wide = torch.full((900, 1304 + 8), 7, device=device, dtype=torch.bfloat16)
     view = wide[:, :1300]
-    launch(glu_kernel, xr, wr, view, cfg(256, 256, 64, 4, 2, persistent=1, superblock=1), activation=activation)
+    launch(glu_kernel, xr, wr, view, cfg(256, 128, 64, 4, 2, persistent=1, superblock=1), activation=activation)
     assert torch.equal(view, base) and float(wide[:, 1300:].float().min()) == 7.0
 
 
@@ -160,8 +162,9 @@ def test_schedules_at_the_benchmark_size(device):
     a, b = oracle.make_inputs("C5")
     ad, bd = a.to(device), b.to(device)
     want = gemm(ad, bd, cfg(256, 256, 128, 4, 2))
+    assert torch.equal(gemm(ad, bd, cfg(256, 256, 128, 4, 2, superblock=1)), want)
     for extra in SCHEDULES:
-        assert torch.equal(gemm(ad, bd, cfg(256, 256, 128, 4, 2, **extra)), want)
+        assert torch.equal(gemm(ad, bd, cfg(256, 128, 128, 4, 2, **extra)), want)      # integer sums: any tile, same bits
 
 
 @pytest.mark.gpu

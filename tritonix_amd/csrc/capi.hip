@@ -47,10 +47,12 @@ static int64_t lds_bytes_of(const tnx_gemm_args* a) {
   const int nw = a->num_warps > 0 ? a->num_warps : 4;
   const int wgm = nw == 4 ? 2 : (a->block_m > a->block_n ? 4 : 2), wgn = nw / wgm > 0 ? nw / wgm : 1;
   const int wtm = a->block_m / wgm, wtn = a->block_n / wgn;
-  const int mi = (wtm % 32 == 0 && wtn % 32 == 0) ? 32 : 16;
-  const int64_t strips = (int64_t)nw * mi * (wtn * 4 + 16);
-  // the persistent kernel keeps its (smaller) strips beside the ring: 8 KiB per wave
-  if (a->schedule & TNX_SCHED_PERSISTENT) return ring + (int64_t)nw * 8192;
+  const int mi = 16;   // TileCfg::MI
+  const int rows = mi;   // EpiStage::ROWS
+  (void)wtm;
+  const int64_t strips = (int64_t)nw * rows * (wtn * 4 + 16);
+  // the persistent kernel keeps its (smaller) strips beside the ring: MI rows of 256 bytes per wave
+  if (a->schedule & TNX_SCHED_PERSISTENT) return ring + (int64_t)nw * mi * 256;
   return ring > strips ? ring : strips;
 }
 
@@ -71,21 +73,31 @@ static int check_common(const tnx_gemm_args* a) {
   return TNX_OK;
 }
 
-static bool fast_layout(const tnx_gemm_args* a) {
+// Which DMA loader the operands can take: 0 = none (element-wise loader only), 1 = row-major B
+// (stride_bn == 1), 2 = k-contiguous B (stride_bk == 1, the layout of x @ w.t()).  Both need row-major A,
+// 16-byte aligned rows and base pointers and k % block_k == 0.
+static int dma_layout(const tnx_gemm_args* a) {
   const int es = elem_size(a->in_dtype);
   const int vec = 16 / es;
-  if (a->stride_ak != 1 || a->stride_bn != 1) return false;
-  if (a->k % a->block_k != 0 || a->k == 0) return false;
-  if ((a->stride_am * es) % 16 != 0 || (a->stride_bk * es) % 16 != 0) return false;
-  if (a->stride_am < 0 || a->stride_bk < 0) return false;
-  if (((uintptr_t)a->a & 15) || ((uintptr_t)a->b & 15)) return false;
-  if (a->n % vec != 0 || a->n < vec) return false;
+  if (a->stride_ak != 1) return 0;
+  if (a->k % a->block_k != 0 || a->k == 0) return 0;
+  if ((a->stride_am * es) % 16 != 0 || a->stride_am < 0) return 0;
+  if (((uintptr_t)a->a & 15) || ((uintptr_t)a->b & 15)) return 0;
   // per-lane DMA offsets are 32-bit
-  if ((int64_t)a->block_m * a->stride_am * es >= (1ll << 32)) return false;
-  if ((int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es >= (1ll << 32)) return false;
-  return true;
+  if ((int64_t)a->block_m * a->stride_am * es >= (1ll << 32)) return 0;
+  if (a->stride_bn == 1) {
+    if ((a->stride_bk * es) % 16 != 0 || a->stride_bk < 0) return 0;
+    if (a->n % vec != 0 || a->n < vec) return 0;
+    if ((int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es >= (1ll << 32)) return 0;
+    return 1;
+  }
+  if (a->stride_bk == 1) {
+    if ((a->stride_bn * es) % 16 != 0 || a->stride_bn < 0) return 0;
+    if ((int64_t)a->block_n * a->stride_bn * es + (int64_t)a->block_k * es >= (1ll << 32)) return 0;
+    return 2;
+  }
+  return 0;
 }
-
 extern "C" int64_t tnx_gemm_lds_bytes(const tnx_gemm_args* a) {
   if (!a) return -1;
   return lds_bytes_of(a);
@@ -106,7 +118,8 @@ extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
   return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)cut_tiles(a) * (size_t)a->block_m * (size_t)a->block_n * 4;
 }
 
-static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs) {
+static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs, bool* bt = nullptr) {
+  if (bt) *bt = false;
   int st = check_common(a);
   if (st != TNX_OK) return st;
   int64_t lds = lds_bytes_of(a);
@@ -131,11 +144,13 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   if (!e) return TNX_E_UNSUPPORTED;
   tnx_gemm_args tmp = *a;
   if (!inspect_ptrs) { tmp.a = nullptr; tmp.b = nullptr; }
-  bool f = fast_layout(&tmp);
+  const int layout = dma_layout(&tmp);
+  bool f = layout == 1 || (layout == 2 && e->fast_bt);
   if (!f && !e->generic) return TNX_E_UNSUPPORTED;
   if (a->schedule & TNX_SCHED_PERSISTENT) {
-    if (!e->persist || !f || a->split_k != 1 || a->k < (int64_t)a->num_stages * a->block_k) return TNX_E_UNSUPPORTED;
+    if (!e->persist || layout != 1 || a->split_k != 1 || a->k < (int64_t)a->num_stages * a->block_k) return TNX_E_UNSUPPORTED;
   }
+  if (bt) *bt = f && layout == 2;
   int64_t tiles = ((a->m + a->block_m - 1) / a->block_m) * ((a->n + a->block_n - 1) / a->block_n);
   if (tiles * a->split_k > 0x7fffffffll) return TNX_E_UNSUPPORTED;
   if (cut_tiles(a) > WS_MAX_TILES) return TNX_E_UNSUPPORTED;  // one arrival counter per cut tile
@@ -166,8 +181,8 @@ extern "C" int tnx_gemm_supported(const tnx_gemm_args* a) { return supported_imp
 
 extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   const KernelEntry* e = nullptr;
-  bool fast = false;
-  int st = supported_impl(a, &e, &fast, true);
+  bool fast = false, bt = false;
+  int st = supported_impl(a, &e, &fast, true, &bt);
   if (st != TNX_OK) return st;
   if (!a->a || !a->b || !a->c) {
     if (a->m == 0 || a->n == 0) return TNX_OK;
@@ -216,7 +231,7 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
     err = e->persist(p, (unsigned)(tiles < cus ? tiles : cus), stream);
   } else {
     unsigned grid = a->split_k > 1 ? (unsigned)(p.split_tile0 + ncut * a->split_k) : (unsigned)(p.tiles_m * p.tiles_n);
-    err = (fast ? e->fast : e->generic)(p, grid, stream);
+    err = (bt ? e->fast_bt : fast ? e->fast : e->generic)(p, grid, stream);
   }
   if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
 
@@ -298,7 +313,7 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     tnx_gemm_args t = *a;   // a and b, when given, count with their base alignment (null = aligned)
     if (t.stride_ak == 0 && t.stride_bn == 0) { t.stride_am = t.k; t.stride_ak = 1; t.stride_bk = t.n; t.stride_bn = 1; }
     t.block_m = 128; t.block_n = 128; t.block_k = bk;
-    dma_ok = fast_layout(&t);
+    dma_ok = dma_layout(&t) != 0;     // every tile the choice below proposes is built for both DMA layouts
   }
   if (a->m <= 64 && dma_ok) {
     // skinny: B is streamed once; K is split until every CU owns one workgroup (measured on the
@@ -396,6 +411,7 @@ extern "C" const char* tnx_kernel_name(int idx) {
       const char* dn = e.dtype == TNX_F16 ? "f16" : e.dtype == TNX_BF16 ? "bf16" : "i8";
       snprintf(buf, sizeof(buf), "%s %d %d %d %d %d%s%s", dn, e.bm, e.bn, e.bk, e.nw, e.stages, e.generic ? " generic" : "",
                e.persist ? " persistent" : "");
+      if (e.fast_bt) strncat(buf, " bt", sizeof(buf) - strlen(buf) - 1);
       return buf;
     }
     idx -= g[i].count;

@@ -194,6 +194,17 @@ __device__ __forceinline__ void dma16(const uint8_t* sbase, uint32_t voff, uint3
                : "memory");
 }
 
+// The same load in two parts, so that a useful instruction (an LDS read) can take the place of the wait
+// state the hardware needs between the write of M0 and the load that uses it.  Nothing that reads or
+// writes M0 may be placed between the two.
+__device__ __forceinline__ void dma16_set_m0(uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0" : : "s"(lds_base) : "memory");
+}
+template <bool NT> __device__ __forceinline__ void dma16_go(const uint8_t* sbase, uint32_t voff) {
+  if (NT) asm volatile("global_load_lds_dwordx4 %0, %1 nt" : : "v"(voff), "s"(sbase) : "memory");
+  else asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase) : "memory");
+}
+
 // same, with the non-temporal hint: for an operand that is streamed from HBM once and never reused
 __device__ __forceinline__ void dma16_nt(const uint8_t* sbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
@@ -272,11 +283,12 @@ struct TileCfg {
   static constexpr int WGM = (NW == 4) ? 2 : (BM > BN ? 4 : 2);  // wave grid
   static constexpr int WGN = NW / WGM;
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;            // wave tile
-#ifdef TNX_EXP_MI16
+  // MFMA shape: 16x16 (x32 for 16-bit, x64 for int8).  With operands that toggle like real data the part runs
+  // against its board-power limit, and per multiply-add the 16x16 instructions draw measurably less than the
+  // 32x32 ones (an MFMA-only loop on random registers sustains 11-15 % more with them, for all three types),
+  // which outweighs their four points of extra issue overhead.  The 32x32 code paths below stay usable
+  // (MI = 32 needs WTM % 32 == 0 && WTN % 32 == 0).
   static constexpr int MI = 16;
-#else
-  static constexpr int MI = (WTM % 32 == 0 && WTN % 32 == 0) ? 32 : 16;
-#endif
   static constexpr int TM = WTM / MI, TN = WTN / MI;
   static constexpr int KB = (MI == 32) ? 32 : 64;                 // k bytes one MFMA consumes
   static constexpr int MMA_K = KB / ES;
@@ -333,7 +345,11 @@ template <> struct OutOf<TagI8> { typedef int type; };
 // 32-bit values, rows padded by 16 bytes to spread the banks.
 template <class C> struct EpiStage {
   static constexpr int PITCH = C::WTN * 4 + 16;
-  static constexpr int WAVE_BYTES = C::MI * PITCH;
+  // row-blocks per pass.  Two (32 rows per pass, half as many passes) was measured on the gated 4096x28672x4096
+  // problem and lost 2-3 %: the longer read-back of a pass delays the first stores.
+  static constexpr int RB = 1;
+  static constexpr int ROWS = RB * C::MI;
+  static constexpr int WAVE_BYTES = ROWS * PITCH;
   static constexpr int BYTES = C::NW * WAVE_BYTES;
 };
 
@@ -434,35 +450,41 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
   constexpr int MI = C::MI;
   constexpr int NGRP = C::ACC_N / 4;                    // groups of four consecutive columns per accumulator tile
   constexpr int PITCH = EpiStage<C>::PITCH;
+  constexpr int RB = EpiStage<C>::RB, ROWS = EpiStage<C>::ROWS;   // a pass moves RB row-blocks = ROWS rows
   constexpr int WCOLS = GLU ? C::WTN / 2 : C::WTN;      // output columns of the wave tile
   constexpr int CPRW = WCOLS / PK::OUTV;                // 16-byte output chunks per strip row
-  constexpr int ITERS = (MI * CPRW + 63) / 64;
+  constexpr int ITERS = (ROWS * CPRW + 63) / 64;
   constexpr int UNR = ITERS % 4 == 0 ? 4 : (ITERS % 2 == 0 ? 2 : 1);   // read-back rows in flight together
   static_assert(WCOLS % PK::OUTV == 0, "wave tile too narrow for 16-byte stores");
   raw* cp = (raw*)cbase;
-  const uint32_t wbase = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
+  const uint32_t wbase0 = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
 #pragma unroll
-  for (int i = 0; i < C::TM; ++i) {
-    if (gm0 + i * MI >= m) break;                       // row-blocks past the last row hold nothing
-    if constexpr (!FROM_WS) {
+  for (int i0 = 0; i0 < C::TM; i0 += RB) {
+    if (gm0 + i0 * MI >= m) break;                      // row-blocks past the last row hold nothing
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j)
+    for (int ii = 0; ii < RB; ++ii) {
+      const int i = i0 + ii;
+      const uint32_t wbase = wbase0 + ii * MI * PITCH;
+      if constexpr (!FROM_WS) {
 #pragma unroll
-        for (int g = 0; g < NGRP; ++g)
-          // (typed vector store: __builtin_bit_cast on an ext-vector element reads element 0)
-          *TNX_LDS(acc4, wbase + (j * MI + g * 8) * 4) =
-              acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-    } else {
-      // 32 loads per lane in flight (G groups x ZB slices): the hand-over is latency-bound otherwise
-      const __amdgpu_buffer_rsrc_t win = agent_window(src.base);
-      const uint32_t q0 = (uint32_t)i * (C::TN * NGRP) * 1024u + lane * 16u;
-      const bool row_ok = gm0 + i * MI + lane % MI < m;
-      if (src.nslices <= 2)
-        sum_slices<acc4, 2, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
-      else if (src.nslices <= 4)
-        sum_slices<acc4, 4, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
-      else
-        sum_slices<acc4, 8, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+          for (int g = 0; g < NGRP; ++g)
+            // (typed vector store: __builtin_bit_cast on an ext-vector element reads element 0)
+            *TNX_LDS(acc4, wbase + (j * MI + g * 8) * 4) =
+                acc4{acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+      } else {
+        // 32 loads per lane in flight (G groups x ZB slices): the hand-over is latency-bound otherwise
+        const __amdgpu_buffer_rsrc_t win = agent_window(src.base);
+        const uint32_t q0 = (uint32_t)i * (C::TN * NGRP) * 1024u + lane * 16u;
+        const bool row_ok = gm0 + i * MI + lane % MI < m;
+        if (src.nslices <= 2)
+          sum_slices<acc4, 2, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
+        else if (src.nslices <= 4)
+          sum_slices<acc4, 4, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
+        else
+          sum_slices<acc4, 8, C::TN * NGRP, MI, NGRP>(win, q0, src, wbase, row_ok);
+      }
     }
     // the strip is private to this wave: its own LDS writes are ordered before its reads
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
@@ -475,7 +497,7 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
         const int q = (it0 + u) * 64 + lane;
         int row = q / CPRW;
         const int cc = q % CPRW;
-        if (MI * CPRW % 64 != 0 && row >= MI) row = MI - 1;
+        if (ROWS * CPRW % 64 != 0 && row >= ROWS) row = ROWS - 1;
 #pragma unroll
         for (int x = 0; x < PK::NF / 4; ++x) {
           const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * PK::NF + 4 * x) * 4);
@@ -486,9 +508,9 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
       for (int u = 0; u < UNR; ++u) {
         const int q = (it0 + u) * 64 + lane;
         const int row = q / CPRW, cc = q % CPRW;
-        const int64_t gm = gm0 + i * MI + row;
+        const int64_t gm = gm0 + i0 * MI + row;
         const int64_t gc = gc0 + cc * PK::OUTV;
-        if ((MI * CPRW % 64 != 0 && row >= MI) || gm >= m) continue;
+        if ((ROWS * CPRW % 64 != 0 && row >= ROWS) || gm >= m) continue;
         raw out[PK::OUTV];
         PK::run(f[u], epi, out);
         raw* dst = cp + gm * scm + gc * scn;
@@ -503,57 +525,60 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
         }
       }
     }
-    // the next row-block overwrites the strip: wait for the reads above
+    // the next pass overwrites the strip: wait for the reads above
     __builtin_amdgcn_s_waitcnt(0xC07F);
   }
 }
 
 // Epilogue of the persistent kernel.  The ring is already being refilled with the next tile's
-// first slabs while this runs, so the accumulators pass through a small strip of their own: 8 KiB
-// per wave = 32 rows x 64 accumulator columns (two 32x32 MFMA tiles side by side), rows 256 bytes
-// apart with the 16-byte chunk index XOR-ed with the row, so neither the column-wise writes nor
+// first slabs while this runs, so the accumulators pass through a small strip of their own: per wave
+// MI rows x 64 accumulator columns (64 / MI MFMA tiles side by side), rows 256 bytes apart with the
+// 16-byte chunk index XOR-ed with the row, so neither the column-wise writes nor
 // the row-wise read-back collide on banks.  FULL: the tile lies inside C and C takes 16-byte
 // stores, so the number of store instructions per wave is the compile-time STORES (the caller's
 // vmcnt arithmetic relies on it).
 template <class C> struct PairStrip {
-  static constexpr int WAVE_BYTES = 32 * 256;
+  static constexpr int WAVE_BYTES = C::MI * 256;              // MI rows of 64 accumulator columns
   static constexpr int BYTES = C::NW * WAVE_BYTES;
+  static constexpr int TPP = 64 / C::MI;                      // MFMA tiles side by side in one pass
 };
 template <class T, class C, class O, bool GLU> struct PairEpilogue {
   typedef typename T::acc_s acc_s;
   typedef Pack16<O, acc_s, GLU> PK;
   static constexpr int OCOLS = GLU ? 32 : 64;                 // output columns per pass
   static constexpr int CPRW = OCOLS / PK::OUTV;               // lanes per output row
-  static constexpr int ITERS = 32 * CPRW / 64;
+  static constexpr int ITERS = C::MI * CPRW / 64;
   static constexpr int CH = PK::NF / 4;                       // 16-byte chunks one lane reads back
-  static constexpr int STORES = C::TM * (C::TN / 2) * ITERS;  // store instructions per wave on a FULL tile
+  static constexpr int STORES = C::TM * (C::TN / PairStrip<C>::TPP) * ITERS;  // store instructions per wave on a FULL tile
 };
 template <class T, class C, class O, bool GLU, bool FULL, class ACC>
 __device__ __forceinline__ void epilogue_store_pairs(ACC (&acc)[C::TM][C::TN], uint8_t* cbase, uint32_t strip, int lane,
                                                      int64_t gm0, int64_t gc0, int64_t m, int64_t ncols, int64_t scm,
                                                      int64_t scn, bool vec_ok, int epi) {
-  static_assert(C::MI == 32 && C::TN % 2 == 0, "pair strips need 32x32 MFMA tiles in an even number of columns");
+  constexpr int MI = C::MI, TPP = PairStrip<C>::TPP, NGRP = C::ACC_N / 4;
+  static_assert(C::TN % TPP == 0 && MI * PairEpilogue<T, C, O, GLU>::CPRW >= 64, "a pass is 64 accumulator columns wide");
   typedef PairEpilogue<T, C, O, GLU> E;
   typedef typename E::acc_s acc_s;
   typedef typename E::PK PK;
   typedef typename PK::raw raw;
   typedef acc_s acc4 __attribute__((ext_vector_type(4)));
   raw* cp = (raw*)cbase;
-  const int wrow = lane & 31, wk = lane >> 5;
+  const int wrow = lane % MI, wk = lane / MI;
   const uint32_t wbase = strip + wrow * 256;
 #pragma unroll
   for (int i = 0; i < C::TM; ++i) {
-    if (!FULL && gm0 + i * 32 >= m) break;
+    if (!FULL && gm0 + i * MI >= m) break;
 #pragma unroll
-    for (int jp = 0; jp < C::TN / 2; ++jp) {
+    for (int jp = 0; jp < C::TN / TPP; ++jp) {
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
+      for (int jj = 0; jj < TPP; ++jj)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int c = jj * 8 + g * 2 + wk;                  // chunk of four columns inside the 64-column pass
+        for (int g = 0; g < NGRP; ++g) {
+          // chunk of four columns inside the 64-column pass: tile jj, then the lane's column group
+          const int c = jj * (MI / 4) + g * (64 / MI) + wk;
           *TNX_LDS(acc4, wbase + ((c ^ (wrow & 15)) << 4)) =
-              acc4{acc[i][2 * jp + jj][4 * g + 0], acc[i][2 * jp + jj][4 * g + 1], acc[i][2 * jp + jj][4 * g + 2],
-                   acc[i][2 * jp + jj][4 * g + 3]};
+              acc4{acc[i][TPP * jp + jj][4 * g + 0], acc[i][TPP * jp + jj][4 * g + 1], acc[i][TPP * jp + jj][4 * g + 2],
+                   acc[i][TPP * jp + jj][4 * g + 3]};
         }
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the strip is private to the wave
       acc_s f[E::ITERS][PK::NF];
@@ -571,7 +596,7 @@ __device__ __forceinline__ void epilogue_store_pairs(ACC (&acc)[C::TM][C::TN], u
       for (int it = 0; it < E::ITERS; ++it) {
         const int q = it * 64 + lane;
         const int row = q / E::CPRW, cc = q % E::CPRW;
-        const int64_t gm = gm0 + i * 32 + row;
+        const int64_t gm = gm0 + i * MI + row;
         const int64_t gc = gc0 + jp * E::OCOLS + cc * PK::OUTV;
         raw out[PK::OUTV];
         PK::run(f[it], epi, out);
@@ -668,16 +693,21 @@ __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t*
 }
 
 template <bool B> struct BoolTag { static constexpr bool value = B; };
+template <int V> struct IntTag { static constexpr int value = V; };
 
 // ---------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------
-template <class T, class C, bool FAST, bool PERSIST = false>
+// BT: B is k-contiguous (element (k, n) at b + n * stride_bn + k, the layout of `x @ w.t()` with a
+// row-major weight): its slab sits in LDS as BN rows of BK elements exactly like the A slab, and its
+// fragments are read with plain ds_read_b128 -- no transposing read is needed.
+template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false>
 __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
   constexpr int MI = C::MI, TM = C::TM, TN = C::TN;
   static_assert(C::VALID, "tile configuration not supported by this kernel");
   static_assert(!PERSIST || FAST, "the persistent kernel is built with the DMA loader only");
+  static_assert(!BT || (FAST && C::B_LOADS % NW == 0), "the k-contiguous B variant is built with the DMA loader only");
   typedef Mma<T, MI> MMA;
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
@@ -703,7 +733,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   int split = 0, logical = 0;
   bool cut = false;
   // launch-order id -> tile coordinates
-  auto locate = [&](int id, int* pid_m, int* pid_n) {
+  auto locate = [&](int id, int* pid_m, int* pid_n) __attribute__((always_inline)) {
     if (p.tile_order == 1) {
       superblock_order(id, p.tiles_m, p.tiles_n, pid_m, pid_n);
     } else {
@@ -744,14 +774,14 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   uint32_t a_voff[C::A_LPW], b_voff[C::B_LPW];
   const uint8_t* a_sbase = p.a;
   const uint8_t* b_sbase = p.b;
-  auto place_tile = [&](int tile_m, int tile_n) {
+  auto place_tile = [&](int tile_m, int tile_n) __attribute__((always_inline)) {
     m0 = (int64_t)tile_m * BM;
     n0 = (int64_t)tile_n * BN;
     if (FAST) {
-      const int64_t lda = p.sam, ldb = p.sbk;
+      const int64_t lda = p.sam, ldb = BT ? p.sbn : p.sbk;
       // wave-uniform by construction; say so, so both stay in SGPRs for the DMA's scalar base operand
       a_sbase = uniform_ptr(p.a + (m0 * lda + (int64_t)kt0 * BK) * ES);
-      b_sbase = uniform_ptr(p.b + ((int64_t)kt0 * BK * ldb + n0) * ES);
+      b_sbase = uniform_ptr(BT ? p.b + (n0 * ldb + (int64_t)kt0 * BK) * ES : p.b + ((int64_t)kt0 * BK * ldb + n0) * ES);
       const int64_t mrem = p.m - 1 - m0;  // last valid row inside this tile
 #pragma unroll
       for (int q = 0; q < C::A_LPW; ++q) {
@@ -761,13 +791,22 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         int64_t r = row < mrem ? row : mrem;
         a_voff[q] = (uint32_t)(r * lda * ES + c * 16);
       }
+      const int64_t nrem = p.n - 1 - n0;  // last valid column inside this tile
 #pragma unroll
       for (int q = 0; q < C::B_LPW; ++q) {
         int P = (q * NW + wave) * 64 + lane;
-        int row = P / C::CPR_B, cs = P % C::CPR_B;
-        int c = cs ^ C::swzB(row);
-        if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
-        b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
+        if (BT) {
+          // rows of the slab are columns of B: same chunk layout and swizzle as the A slab
+          int row = P / C::CPR_A, cs = P % C::CPR_A;
+          int c = cs ^ C::swzA(row);
+          int64_t r = row < nrem ? row : nrem;
+          b_voff[q] = (uint32_t)(r * ldb * ES + c * 16);
+        } else {
+          int row = P / C::CPR_B, cs = P % C::CPR_B;
+          int c = cs ^ C::swzB(row);
+          if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
+          b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
+        }
       }
     }
   };
@@ -775,7 +814,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
 
   // element-wise loader: any strides, any ragged edge, zero fill.  Used for
   // the K-tail slab of FAST kernels and for every slab otherwise.
-  auto load_slab_generic = [&](int kt_global, uint32_t stage_base) {
+  auto load_slab_generic = [&](int kt_global, uint32_t stage_base) __attribute__((always_inline)) {
     const int64_t k0 = (int64_t)kt_global * BK;
     for (int idx = tid; idx < BM * BK; idx += C::THREADS) {
       int row = idx / BK, kk = idx % BK;
@@ -808,7 +847,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   };
 
   // one DMA op (q-th of this wave) of local slab t, into ring slot t % STAGES
-  auto dma_op = [&](int q, uint32_t stage_base) {
+  auto dma_op = [&](int q, uint32_t stage_base) __attribute__((always_inline)) {
     if (q < C::A_LPW) {
       dma16(a_sbase, a_voff[q], stage_base + (q * NW + wave) * 1024);
     } else {
@@ -819,11 +858,21 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         dma16(b_sbase, b_voff[q - C::A_LPW], stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
     }
   };
-  auto dma_advance = [&]() {
-    a_sbase += BK * ES;
-    b_sbase += (int64_t)BK * p.sbk * ES;
+  // the same op in two parts (see dma16_set_m0): LDS target first, the load after one other instruction
+  auto dma_target = [&](int q, uint32_t stage_base) __attribute__((always_inline)) {
+    if (q < C::A_LPW) dma16_set_m0(stage_base + (q * NW + wave) * 1024);
+    else dma16_set_m0(stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
   };
-  auto stage_of = [&](int t) { return lds0 + (uint32_t)(t % STAGES) * C::STAGE_BYTES; };
+  auto dma_go = [&](int q) __attribute__((always_inline)) {
+    if (q < C::A_LPW) dma16_go<false>(a_sbase, a_voff[q]);
+    else if (BM <= 64 && p.b_once) dma16_go<true>(b_sbase, b_voff[q - C::A_LPW]);
+    else dma16_go<false>(b_sbase, b_voff[q - C::A_LPW]);
+  };
+  auto dma_advance = [&]() __attribute__((always_inline)) {
+    a_sbase += BK * ES;
+    b_sbase += BT ? (int64_t)BK * ES : (int64_t)BK * p.sbk * ES;
+  };
+  auto stage_of = [&](int t) __attribute__((always_inline)) { return lds0 + (uint32_t)(t % STAGES) * C::STAGE_BYTES; };
 
   // ---- fragment addressing ----------------------------------------------
   const int wy = wave / C::WGN, wx = wave % C::WGN;
@@ -848,6 +897,13 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     b_joff[j] = (uint32_t)(((16 / ES) * b_kg + b_sub) * C::ROWB_B) + (((colb >> 4) ^ b_sw) << 4) + (colb & 15);
   }
 
+  // k-contiguous B: fragment j of k step ks sits at bt_koff[ks] + j * MI rows, read like an A fragment
+  const int bt_row = wx * C::WTN + (lane % MI);
+  uint32_t bt_koff[C::KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < C::KSTEPS; ++ks)
+    bt_koff[ks] = bt_row * C::ROWB_A + (((ks * (C::KB / 16) + a_kg) ^ C::swzA(bt_row)) << 4);
+
   acc_t acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -857,25 +913,27 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // two register sets of fragments: one being multiplied, one being filled
   i32x4 fa[2][TM];
   i32x2 fb[2][TN][2];
-  constexpr int NREAD = 2 * TN + TM, NMMA = TM * TN;
+  i32x4 fbq[2][TN];             // k-contiguous B: one 16-byte read per fragment
+  constexpr int NBREAD = BT ? TN : 2 * TN;
+  constexpr int NREAD = NBREAD + TM, NMMA = TM * TN;
   constexpr int RPM = (NREAD + NMMA - 1) / NMMA;        // LDS reads slotted behind each MFMA
   constexpr int DPM = (C::LPW + NMMA - 1) / NMMA;       // DMA ops slotted behind each MFMA
 
-  auto read_one = [&](int set, int idx, uint32_t sa, uint32_t sb, int ks) {
-    if (idx < 2 * TN) {
+  auto read_one = [&](int set, int idx, uint32_t sa, uint32_t sb, int ks) __attribute__((always_inline)) {
+    if (BT && idx < NBREAD) {
+      fbq[set][idx] = *TNX_LDS(i32x4, sb + bt_koff[ks] + idx * MI * C::ROWB_A);
+    } else if (idx < NBREAD) {
       int j = idx >> 1, h = idx & 1;
       fb[set][j][h] = lds_read_tr<ES>(sb + b_joff[j] + ks * C::MMA_K * C::ROWB_B + h * RPR * C::ROWB_B);
     } else {
-      int i = idx - 2 * TN;
+      int i = idx - NBREAD;
       fa[set][i] = *TNX_LDS(i32x4, sa + a_koff[ks] + i * MI * C::ROWB_A);
     }
   };
-  auto mma_one = [&](int set, int idx) {
+  auto mma_one = [&](int set, int idx) __attribute__((always_inline)) {
     int i = idx / TN, j = idx % TN;
-#ifdef TNX_EXP_SERP
-    if (i & 1) j = TN - 1 - j;
-#endif
-    i32x4 b4 = i32x4{fb[set][j][0].x, fb[set][j][0].y, fb[set][j][1].x, fb[set][j][1].y};
+    if (i & 1) j = TN - 1 - j;   // serpentine walk of the wave's MFMA tiles: one operand changes per instruction, never both
+    i32x4 b4 = BT ? fbq[set][j] : i32x4{fb[set][j][0].x, fb[set][j][0].y, fb[set][j][1].x, fb[set][j][1].y};
     acc[i][j] = MMA::run(b4, fa[set][i], acc[i][j]);   // rows = n, cols = m: the tile comes out transposed
   };
 
@@ -895,67 +953,72 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // straight-line code.
   constexpr int PERIOD = C::KSTEPS * NMMA;                       // MFMA slots per period
   // slots the refill is spread over.  Two-slab rings: the refill is due at the next barrier, so it
-  // is front-loaded; with one wave per SIMD a single k step of DMA issue backs up the texture
-  // address queue (measured: 2630 -> 2210 cycles per slab when spread over two), with two waves
-  // per SIMD the other wave already covers the stall.
-  constexpr int SPAN2 = (NW == 4 && 2 * NMMA <= PERIOD) ? 2 * NMMA : NMMA;
+  // is front-loaded: over the first half of the period with one wave per SIMD (a shorter burst backs
+  // up the texture address queue and stalls the wave; spread over the whole period the last loads
+  // are waited for as soon as they are issued), over the first quarter with two waves per SIMD
+  // (the other wave covers the stall).
+  constexpr int SPAN2 = (NW == 4 ? PERIOD / 2 : PERIOD / 4) > 0 ? (NW == 4 ? PERIOD / 2 : PERIOD / 4) : 1;
   constexpr int SPAN = (STAGES == 2 || !FAST) ? SPAN2 : PERIOD;
   constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
   constexpr int NEXT0 = C::KSTEPS & 1;                           // set that receives step 0 of the next slab
 
-  // DMA ops due at period slot `slot` (compile-time after unrolling)
-  auto dma_slot = [&](int slot, uint32_t dst) {
-    if (slot < SPAN) {
-      const int lo = slot * C::LPW / SPAN, hi = (slot + 1) * C::LPW / SPAN;
+  // One MFMA slot: the MFMA, then the LDS reads and DMA ops slotted behind it.  When exactly one DMA op and at
+  // least one read are due, the read sits between the op's M0 write and its load (it fills the wait state).
+  auto slot_body = [&](int mset, int x, int rset, int& rd, uint32_t sa, uint32_t sb, int ks_next, bool with_dma, int slot,
+                       uint32_t dst) __attribute__((always_inline)) {
+    mma_one(mset, x);
+    int lo = 0, hi = 0;
+    if (with_dma && slot < SPAN) { lo = slot * C::LPW / SPAN; hi = (slot + 1) * C::LPW / SPAN; }
+    const bool paired = hi - lo == 1 && rd < NREAD;
+    if (paired) dma_target(lo, dst);
+#pragma unroll
+    for (int q = 0; q < RPM; ++q)
+      if (rd < NREAD) { read_one(rset, rd, sa, sb, ks_next); ++rd; }
+    if (paired) dma_go(lo);
+    else
 #pragma unroll
       for (int q = lo; q < hi; ++q) dma_op(q, dst);
-    }
+    __builtin_amdgcn_sched_barrier(0);
   };
-  // k steps 0 .. KSTEPS-2 of the slab at (sa, sb): multiply register set (ks & 1) while filling
-  // the other set with step ks+1; WITH_DMA: keep issuing the refill into slot `dst`
-  auto inner_steps = [&](uint32_t sa, uint32_t sb, auto with_dma, uint32_t dst) {
+  // `par` (0 or 1, compile-time) is added to every register-set index: with an odd number of k steps per slab
+  // the two sets trade roles from one slab to the next, and the unrolled bulk of the K loop follows that by
+  // alternating par; where the slab index is a run-time value (par = 0) the sets are swapped by copying.
+  auto inner_steps = [&](uint32_t sa, uint32_t sb, auto with_dma, uint32_t dst, auto par) __attribute__((always_inline)) {
     constexpr bool WITH_DMA = decltype(with_dma)::value;
+    constexpr int P = decltype(par)::value;
 #pragma unroll
     for (int ks = 0; ks + 1 < C::KSTEPS; ++ks) {
       int rd = 0;
 #pragma unroll
-      for (int x = 0; x < NMMA; ++x) {
-        mma_one(ks & 1, x);
-#pragma unroll
-        for (int q = 0; q < RPM; ++q)
-          if (rd < NREAD) { read_one((ks + 1) & 1, rd, sa, sb, ks + 1); ++rd; }
-        if constexpr (WITH_DMA) dma_slot(NMMA + ks * NMMA + x, dst);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int x = 0; x < NMMA; ++x)
+        slot_body((ks + P) & 1, x, (ks + 1 + P) & 1, rd, sa, sb, ks + 1, WITH_DMA, NMMA + ks * NMMA + x, dst);
     }
   };
   // last k step of the slab whose fragments sit in set LAST; prefetches step 0 of the slab at (sa1, sb1)
-  auto last_step = [&](uint32_t sa1, uint32_t sb1, auto with_dma, uint32_t dst) {
+  // (`par` is the parity of the slab that is ending; `swap`: bring the sets back to par = 0 by copying)
+  auto last_step = [&](uint32_t sa1, uint32_t sb1, auto with_dma, uint32_t dst, auto par, auto swap) __attribute__((always_inline)) {
     constexpr bool WITH_DMA = decltype(with_dma)::value;
+    constexpr int P = decltype(par)::value;
     int rd = 0;
 #pragma unroll
-    for (int x = 0; x < NMMA; ++x) {
-      mma_one(LAST, x);
-#pragma unroll
-      for (int q = 0; q < RPM; ++q)
-        if (rd < NREAD) { read_one(NEXT0, rd, sa1, sb1, 0); ++rd; }
-      if constexpr (WITH_DMA) dma_slot(x, dst);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (C::KSTEPS & 1) {   // odd KSTEPS: the two register sets trade roles every slab
+    for (int x = 0; x < NMMA; ++x) slot_body((LAST + P) & 1, x, (NEXT0 + P) & 1, rd, sa1, sb1, 0, WITH_DMA, x, dst);
+    if ((C::KSTEPS & 1) && decltype(swap)::value) {   // odd KSTEPS: the two register sets trade roles every slab
 #pragma unroll
       for (int i = 0; i < TM; ++i) { i32x4 tmp = fa[0][i]; fa[0][i] = fa[1][i]; fa[1][i] = tmp; }
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int h = 0; h < 2; ++h) { i32x2 tmp = fb[0][j][h]; fb[0][j][h] = fb[1][j][h]; fb[1][j][h] = tmp; }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) { i32x4 tmp = fbq[0][j]; fbq[0][j] = fbq[1][j]; fbq[1][j] = tmp; }
     }
   };
   typedef BoolTag<true> Yes;
   typedef BoolTag<false> No;
+  typedef IntTag<0> Par0;
 
   // first STAGES slabs of the tile the loader stands on
-  auto issue_prologue = [&]() {
+  auto issue_prologue = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < STAGES; ++s) {
       if (s < KT) {
@@ -970,13 +1033,13 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
   };
   // the K loop of one tile, from "slab 0 has landed" to the last MFMA; the prologue has been issued
-  auto k_loop = [&]() {
+  auto k_loop = [&]() __attribute__((always_inline)) {
   if (KT > 0) {
     __syncthreads();
     const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
 #pragma unroll
     for (int r = 0; r < NREAD; ++r) read_one(0, r, sa, sb, 0);
-    inner_steps(sa, sb, No{}, 0u);
+    inner_steps(sa, sb, No{}, 0u, Par0{});
   }
 
   int t = 0;
@@ -984,19 +1047,36 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // STAGES periods per trip so every ring slot is a compile-time constant there (LDS addresses
   // become instruction immediates, DMA targets become scalar constants); what is left over runs
   // with run-time slots.
+  // With an odd number of k steps per slab the trip covers an even number of periods, so that the register
+  // sets are back in their starting roles at the end of every trip without a copy.
   if constexpr (FAST) {
-    for (; t + 2 * STAGES - 1 < KT; t += STAGES) {
-#pragma unroll
-      for (int j = 0; j < STAGES; ++j) {
+    constexpr int U = ((C::KSTEPS & 1) && (STAGES & 1)) ? 2 * STAGES : STAGES;
+    for (; t + U + STAGES - 1 < KT; t += U) {
+      auto period = [&](auto jtag) __attribute__((always_inline)) {
+        constexpr int j = decltype(jtag)::value;
+        constexpr int P = (C::KSTEPS & 1) ? (j & 1) : 0;          // parity of the slab whose last k step runs now
         __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        const uint32_t dst = lds0 + (uint32_t)j * C::STAGE_BYTES;
+        const uint32_t dst = lds0 + (uint32_t)(j % STAGES) * C::STAGE_BYTES;
         const uint32_t sa1 = lds0 + (uint32_t)((j + 1) % STAGES) * C::STAGE_BYTES, sb1 = sa1 + C::A_BYTES;
-        last_step(sa1, sb1, Yes{}, dst);
-        inner_steps(sa1, sb1, Yes{}, dst);
+        last_step(sa1, sb1, Yes{}, dst, IntTag<P>{}, No{});
+        inner_steps(sa1, sb1, Yes{}, dst, IntTag<(C::KSTEPS & 1) ? (P ^ 1) : 0>{});
         dma_advance();
-      }
+      };
+      static_assert(U <= 12, "unroll table below covers twelve periods");
+      period(IntTag<0>{});
+      if constexpr (U > 1) period(IntTag<1>{});
+      if constexpr (U > 2) period(IntTag<2>{});
+      if constexpr (U > 3) period(IntTag<3>{});
+      if constexpr (U > 4) period(IntTag<4>{});
+      if constexpr (U > 5) period(IntTag<5>{});
+      if constexpr (U > 6) period(IntTag<6>{});
+      if constexpr (U > 7) period(IntTag<7>{});
+      if constexpr (U > 8) period(IntTag<8>{});
+      if constexpr (U > 9) period(IntTag<9>{});
+      if constexpr (U > 10) period(IntTag<10>{});
+      if constexpr (U > 11) period(IntTag<11>{});
     }
   }
   for (; t + STAGES < KT; ++t) {
@@ -1007,12 +1087,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
     if constexpr (FAST) {
-      last_step(sa1, sb1, Yes{}, dst);
-      inner_steps(sa1, sb1, Yes{}, dst);
+      last_step(sa1, sb1, Yes{}, dst, Par0{}, Yes{});
+      inner_steps(sa1, sb1, Yes{}, dst, Par0{});
       dma_advance();
     } else {
-      last_step(sa1, sb1, No{}, 0u);
-      inner_steps(sa1, sb1, No{}, 0u);
+      last_step(sa1, sb1, No{}, 0u, Par0{}, Yes{});
+      inner_steps(sa1, sb1, No{}, 0u, Par0{});
     }
   }
   // (2) ring draining: nothing left to issue
@@ -1021,8 +1101,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
-    last_step(sa1, sb1, No{}, 0u);
-    inner_steps(sa1, sb1, No{}, 0u);
+    last_step(sa1, sb1, No{}, 0u, Par0{}, Yes{});
+    inner_steps(sa1, sb1, No{}, 0u, Par0{});
   }
   // (3) last k step of the final slab
   if (KT > 0) {
@@ -1100,12 +1180,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         place_tile(nm, nn);
         issue_prologue();
       }
+      // The epilogue's per-lane offsets depend only on the lane: left alone, the compiler computes them once
+      // before the tile loop and keeps them in registers across every K loop, which spills.  An opaque copy of
+      // the lane index ties them to this iteration.
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
       if (!glu) {
-        if (full) epilogue_store_pairs<T, C, O, false, true>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, true, 0);
-        else epilogue_store_pairs<T, C, O, false, false>(acc, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+        if (full) epilogue_store_pairs<T, C, O, false, true>(acc, p.c, strip, lane_e, gm0, gn0, p.m, p.n, p.scm, p.scn, true, 0);
+        else epilogue_store_pairs<T, C, O, false, false>(acc, p.c, strip, lane_e, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
       } else {
-        if (full) epilogue_store_pairs<T, C, O, true, true>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, true, p.epilogue);
-        else epilogue_store_pairs<T, C, O, true, false>(acc, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
+        if (full) epilogue_store_pairs<T, C, O, true, true>(acc, p.c, strip, lane_e, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, true, p.epilogue);
+        else epilogue_store_pairs<T, C, O, true, false>(acc, p.c, strip, lane_e, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn, p.c_vec_ok, p.epilogue);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)

@@ -15,6 +15,7 @@ struct KernelEntry {
   launch_fn fast;     // DMA loader: row-major, 16-byte aligned, k % bk == 0
   launch_fn generic;  // element-wise loader: any strides / ragged k; may be null
   launch_fn persist;  // DMA loader, one workgroup per CU walking its tiles; may be null
+  launch_fn fast_bt;  // DMA loader for k-contiguous B (stride_bk == 1, the `x @ w.t()` layout); may be null
 };
 
 struct KernelGroup {
@@ -22,18 +23,20 @@ struct KernelGroup {
   int count;
 };
 
-template <class T, class C, bool FAST, bool PERSIST = false>
+template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false>
 hipError_t launch_tile(const GemmParams& p, unsigned grid, hipStream_t stream) {
   static_assert(C::VALID, "tile configuration is not buildable");
-  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST, PERSIST>), dim3(grid), dim3(C::THREADS), 0, stream, p);
+  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST, PERSIST, BT>), dim3(grid), dim3(C::THREADS), 0, stream, p);
   return hipGetLastError();
 }
 
-// The persistent variant exists for the large four-wave tiles whose ring leaves room for the
-// epilogue's own strips (8 KiB per wave) inside the 160 KiB of one CU.
+// The persistent variant exists for the four-wave tiles from 128x128 to 256x128 / 128x256: their ring leaves
+// room for the epilogue's own strips (MI rows of 256 bytes per wave) inside the 160 KiB of one CU, and a wave's
+// accumulators take at most 128 registers, so the state the tile loop carries still fits the register file
+// (with the 256 accumulator registers of a 256x256 tile it does not: the compiler spills inside the K loop).
 template <class C> constexpr bool persist_ok() {
-  return C::NW == 4 && C::BM >= 128 && C::BN >= 128 && C::MI == 32 && C::TN % 2 == 0 &&
-         C::LDS_BYTES + PairStrip<C>::BYTES <= 163840;
+  return C::NW == 4 && C::BM >= 128 && C::BN >= 128 && C::TN % PairStrip<C>::TPP == 0 &&
+         C::TM * C::TN * C::ACC_N <= 128 && C::LDS_BYTES + PairStrip<C>::BYTES <= 163840;
 }
 template <class T, class C, bool OK = persist_ok<C>()> struct PersistLaunch {
   static constexpr launch_fn fn = nullptr;
@@ -48,10 +51,20 @@ launch_fn skinny_lookup(int dtype, int ring);
 constexpr int SKINNY_BM = 16, SKINNY_BN = 32, SKINNY_BK = 32, SKINNY_NW = 8, SKINNY_SPLIT = 8;
 constexpr int SKINNY_STEP_BYTES = 3072;
 
+// The k-contiguous-B variant exists for the tiles whose K slab is one 128-byte line per row (the tiles the
+// built-in choice uses).
+template <class C> constexpr bool bt_ok() { return C::BK * C::ES == 128; }
+template <class T, class C, bool OK = bt_ok<C>()> struct BtLaunch {
+  static constexpr launch_fn fn = nullptr;
+};
+template <class T, class C> struct BtLaunch<T, C, true> {
+  static constexpr launch_fn fn = &launch_tile<T, C, true, false, true>;
+};
+
 #define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
   {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
    &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \
    GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr,               \
-   PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
+   PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn, BtLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
 
 }  // namespace tnx

@@ -175,13 +175,19 @@ def save_tuned(op: str, key: tuple, cfg: dict) -> None:
         pass
 
 
-def dma_layout(a, b) -> bool:
-    """True when the operands can take the direct-to-LDS loader: row-major A and B, 16-byte aligned rows and base
-    pointers.  Most tile kernels are built with that loader only, so it is part of every config-memo key."""
+def dma_layout(a, b) -> int:
+    """Layout class of the operands, part of every config-memo key: 1 = row-major A and B, 2 = row-major A and
+    k-contiguous B (``w.t()`` of a row-major weight), both with 16-byte aligned rows and base pointers -- the two
+    layouts the direct-to-LDS loaders take; 0 = anything else (the two tiles built with the element-wise loader)."""
     es = a.element_size()
-    return bool(a.stride(1) == 1 and b.stride(1) == 1 and a.stride(0) >= 0 and b.stride(0) >= 0
-                and (a.stride(0) * es) % 16 == 0 and (b.stride(0) * es) % 16 == 0
-                and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0 and b.shape[1] % (16 // es) == 0)
+    if not (a.stride(1) == 1 and a.stride(0) >= 0 and (a.stride(0) * es) % 16 == 0
+            and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0):
+        return 0
+    if b.stride(1) == 1 and b.stride(0) >= 0 and (b.stride(0) * es) % 16 == 0 and b.shape[1] % (16 // es) == 0:
+        return 1
+    if b.stride(0) == 1 and b.stride(1) >= 0 and (b.stride(1) * es) % 16 == 0:
+        return 2
+    return 0
 
 
 def _tuned_or_tune(op: str, key: tuple, kernel, launcher, fallback):
