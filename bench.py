@@ -21,6 +21,8 @@ Switches for profiling and for the clock / power evidence:
   --operands zeros   all-zero operands of the same shapes: the same instruction stream without data-dependent
                      switching power, so the shader clock stays at its maximum (results are then trivially zero)
   --splitk-reduce atomic   C3 with the K slices added by fp32 atomics instead of the ordered hand-over (for the A/B)
+  --mfma-ceiling     time tnx_probe_mfma: nothing but MFMAs on register operands, 16x16 and 32x32 tiles, random and
+                     all-zero operands; what the pipes sustain on this board before any data is moved ("mfma_ceiling")
   --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
                      socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
@@ -59,6 +61,8 @@ def parse():
     ap.add_argument("--operands", choices=("random", "zeros"), default="random")
     ap.add_argument("--splitk-reduce", choices=("ordered", "atomic"), default="ordered",
                     help="C3 only: how the K slices meet (ordered = stored apart, summed in slice order; atomic = fp32 atomic adds)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="also time the MFMA-only loop (no data movement) for both MFMA shapes and both operand kinds")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -184,6 +188,35 @@ def sustain(step, seconds, flops):
     return out
 
 
+def mfma_ceiling(torch, dev, dtype_code, peak):
+    """T(FL)OP/s of the MFMA-only loop: {"16x16": {"random": .., "zeros": ..}, "32x32": {...}} (same protocol as the
+    kernels: pre-roll, then one HIP-event pair around back-to-back launches on the launch stream)."""
+    import ctypes
+
+    from tritonix_amd import _C
+
+    lib = _C.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    scratch = torch.empty(cus * 256, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    ops = ctypes.c_double()
+    out = {}
+    for rows in (16, 32):
+        for kind, zero in (("random", 0), ("zeros", 1)):
+            def launch(_i=0):
+                st = lib.tnx_probe_mfma(dtype_code, rows, zero, cus, 2000, scratch.data_ptr(), scratch.numel() * 4, stream,
+                                        ctypes.byref(ops))
+                assert st == _C.OK, _C.strerror(st)
+            for _ in range(30):
+                launch()
+            torch.cuda.synchronize()
+            ms = region_time(launch, 40)
+            out.setdefault(f"{rows}x{rows}", {})[kind] = round(ops.value / ms / 1e9, 1)
+    out["peak"] = peak
+    out["frac_of_peak_random_16x16"] = round(out["16x16"]["random"] / peak, 4)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -241,6 +274,9 @@ def main():
     ok = True
     if "C2" in only:
         ok = headline(torch, dev, oracle, mm, args, operands, out)
+    if args.mfma_ceiling:
+        out["mfma_ceiling"] = {"bf16": mfma_ceiling(torch, dev, _C.BF16, PEAK["bf16"]),
+                               "i8": mfma_ceiling(torch, dev, _C.I8, PEAK["i8"])}
     extras_wanted = [s for s in only if s != "C2"]
     if extras_wanted:
         out["per_config"] = extras(torch, dev, oracle, mm, sg, args, operands, extras_wanted)

@@ -172,6 +172,16 @@ int tnx_tile_coords(int schedule, int id, int tiles_m, int tiles_n, int group_m,
 int tnx_kernel_count(void);
 const char* tnx_kernel_name(int i);
 
+/* Measurement aid with no counterpart in the reference: launch a kernel of `workgroups` x 4 waves that issues
+ * nothing but MFMAs of `dtype` (TNX_F16 / TNX_BF16 / TNX_I8) on operands held in registers -- 16x16 (mfma_rows =
+ * 16) or 32x32 (32) tiles, `iterations` x 64 (resp. 32) instructions per wave, operands random (data-like
+ * switching activity) or all zero.  The rate it reaches is what the MFMA pipes sustain on this board before any
+ * operand has been moved: with random operands it is set by the board's power limit and bounds every GEMM kernel
+ * from above.  `scratch` receives workgroups * 1024 bytes of don't-care output; *ops_per_launch (may be NULL) the
+ * multiply-add count x 2.  Asynchronous on `stream`; timing is the caller's. */
+int tnx_probe_mfma(int dtype, int mfma_rows, int zero_operands, int workgroups, int iterations, void* scratch,
+                   size_t scratch_bytes, void* stream, double* ops_per_launch);
+
 const char* tnx_strerror(int status);
 int tnx_last_hip_error(void); /* hipError_t of the last TNX_E_HIP on this thread */
 int tnx_version(void);

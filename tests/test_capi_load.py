@@ -160,7 +160,7 @@ def test_default_config_of_the_benchmark_shapes():
 
     picked = []
     assert pick(_C.BF16, _C.BF16, 8192, 8192, 8192) == (256, 256, 64, 4, 2, 1, 0)
-    assert pick(_C.BF16, _C.BF16, 4096, 28672, 4096) == (256, 256, 64, 4, 2, 1, 0)
+    assert pick(_C.BF16, _C.BF16, 4096, 28672, 4096) == (256, 256, 64, 8, 2, 1, 0)     # short K loop: two waves per SIMD
     assert pick(_C.I8, _C.I32, 8192, 8192, 8192) == (256, 256, 128, 4, 2, 1, 0)
     assert pick(_C.F16, _C.F16, 1024, 768, 512) == (64, 64, 64, 4, 4, 1, 0)
     assert pick(_C.BF16, _C.BF16, 16, 4096, 14336) == (64, 128, 64, 8, 3, 8, 0)

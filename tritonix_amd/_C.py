@@ -27,7 +27,7 @@ OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP, E_STATIC_LIMIT = 0, 1, 
 STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
-           "tnx_gemm_default_config", "tnx_tile_coords", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
+           "tnx_gemm_default_config", "tnx_tile_coords", "tnx_probe_mfma", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
            "tnx_last_hip_error", "tnx_version")
 
 
@@ -76,6 +76,9 @@ def load() -> ctypes.CDLL:
     lib.tnx_gemm_default_config.restype = ctypes.c_int
     lib.tnx_tile_coords.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_int)] * 2
     lib.tnx_tile_coords.restype = ctypes.c_int
+    lib.tnx_probe_mfma.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                                        ctypes.POINTER(ctypes.c_double)]
+    lib.tnx_probe_mfma.restype = ctypes.c_int
     lib.tnx_kernel_count.argtypes = []
     lib.tnx_kernel_count.restype = ctypes.c_int
     lib.tnx_kernel_name.argtypes = [ctypes.c_int]
