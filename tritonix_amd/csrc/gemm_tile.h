@@ -313,13 +313,18 @@ struct TileCfg {
     return CPR_A >= 8 ? ((row & 7) ^ ((row >> 3) & 1)) : (((row >> 1) & 3) ^ ((row >> 3) & 1));
   }
   // chunk-index XOR applied to row `row` (a k index) of the B slab
+  // (A transposing read serves the four 16-lane groups of a wave in two passes; with 16x16 MFMA tiles the two
+  // groups of a pass read the same columns 8 k rows apart (16 for int8), so one more row bit enters the XOR to
+  // keep them on different banks: it moves the second group onto exactly the chunk slots the first leaves free.)
   static __host__ __device__ constexpr int swzB(int row) {
     if (ES == 2) {
-      if (CPR_B >= 16) { int k = row & 3; return (2 * k + (k >> 1)) << 1; }
-      return (row & 3) << 1;
+      const int pass = MI == 16 ? (((row >> 3) ^ (row >> 4)) & 1) << 1 : 0;
+      if (CPR_B >= 16) { int k = row & 3; return ((2 * k + (k >> 1)) << 1) ^ pass; }
+      return ((row & 3) << 1) ^ pass;
     } else {
-      if (CPR_B >= 16) { int k = row & 7; return 2 * k + (k >> 2); }
-      return row & 7;
+      const int pass = MI == 16 ? ((row >> 4) ^ (row >> 5)) & 1 : 0;
+      if (CPR_B >= 16) { int k = row & 7; return (2 * k + (k >> 2)) ^ pass; }
+      return (row & 7) ^ pass;
     }
   }
 };
@@ -889,7 +894,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int b_sub = (ES == 2) ? (li >> 2) : (li >> 1);               // k row inside the transposed block
   const int b_colb0 = (wx * C::WTN + ((MI == 32) ? 16 * (blk & 1) : 0)) * ES + ((ES == 2) ? 8 * (li & 3) : 8 * (li & 1));
   constexpr int RPR = 8 / ES;                                       // k rows one transposing read covers
-  const int b_sw = C::swzB(b_sub);
+  const int b_sw = C::swzB((16 / ES) * b_kg + b_sub);     // the same for every k step and both halves of a fragment
   uint32_t b_joff[TN];          // byte offset inside the B slab, per column block
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -953,10 +958,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // straight-line code.
   constexpr int PERIOD = C::KSTEPS * NMMA;                       // MFMA slots per period
   // slots the refill is spread over.  Two-slab rings: the refill is due at the next barrier, so it
-  // is front-loaded: over the first half of the period with one wave per SIMD (a shorter burst backs
-  // up the texture address queue and stalls the wave; spread over the whole period the last loads
-  // are waited for as soon as they are issued), over the first quarter with two waves per SIMD
-  // (the other wave covers the stall).
+  // is front-loaded: over the first half of the period with one wave per SIMD (measured on 8192^3,
+  // bf16 256x256x64: a quarter of the period 477, three eighths 853, half 1430, three quarters
+  // 1380 TFLOP/s -- a faster burst backs up the texture address path and stalls the wave for far
+  // longer than it saves; spread further, the last loads are waited for as soon as they are
+  // issued), over the first quarter with two waves per SIMD (the other wave covers the stall).
   constexpr int SPAN2 = (NW == 4 ? PERIOD / 2 : PERIOD / 4) > 0 ? (NW == 4 ? PERIOD / 2 : PERIOD / 4) : 1;
   constexpr int SPAN = (STAGES == 2 || !FAST) ? SPAN2 : PERIOD;
   constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
