@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the tiled-GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune] [--only C2,C5] [--operands random|zeros]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tune] [--only C2,C5,CONV] [--operands random|zeros]
                     [--sustain SECONDS] [--no-extras] [--no-cpu] [--no-vendor]
 
 A step is one launch of the headline workload -- the bf16 8192^3 GEMM
@@ -48,7 +48,7 @@ TRAFFIC_KIB_C2 = {"fetch": 792810.7, "fetch_scale": 2.0, "write": 190464.0, "wri
 TRAFFIC_BYTES_C2 = int((TRAFFIC_KIB_C2["fetch"] * TRAFFIC_KIB_C2["fetch_scale"]
                         + TRAFFIC_KIB_C2["write"] * TRAFFIC_KIB_C2["write_scale"]) * 1024)
 
-ALL = ("C2", "C1", "C3", "C4", "C5", "FFN")
+ALL = ("C2", "C1", "C3", "C4", "C5", "FFN", "CONV")
 
 
 def parse():
@@ -495,6 +495,42 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
             r["parity_ok"] = bool(oracle.within_tolerance(y[rows.to(dev)], hidden @ w3_cpu.float())[0])
             del w3, y
         del x, w, z
+
+    # CONV: conv2d forward as an implicit GEMM, a ResNet-style 3x3 layer (batch 32, 256 -> 256 channels, 56x56, padding 1):
+    # GEMM_M = 100352 pixels, GEMM_N = 256, GEMM_K = 2304.  Algorithmic bytes: input + weight + bias + output once.
+    if "CONV" in wanted:
+        from tritonix_amd.ops.conv2d import conv2d_forward, torch_conv2d_forward
+        import tritonix_amd.ops.conv2d.forward as conv
+
+        g = torch.Generator("cpu").manual_seed(66)
+        n_, c_, hw_, k_ = 32, 256, 56, 256
+        x_cpu = torch.randn(n_, c_, hw_, hw_, generator=g).bfloat16()
+        w_cpu = (torch.randn(k_, c_, 3, 3, generator=g) / 48).bfloat16()
+        b_cpu = torch.randn(k_, generator=g).bfloat16()
+        if zeros:
+            x_cpu.zero_(); w_cpu.zero_(); b_cpu.zero_()
+        x, w, b = x_cpu.to(dev), w_cpu.to(dev), b_cpu.to(dev)
+        y = conv2d_forward(x, w, b, (1, 1), (1, 1), (1, 1))          # times the candidate tiles once, as the reference does
+        cfg = next(iter(v for kk, v in conv._CONV_FWD_CONFIG_CACHE.items() if kk[:5] == (n_, c_, hw_, hw_, k_)))
+        flops = 2.0 * n_ * hw_ * hw_ * k_ * c_ * 9
+        bytes_ = 2 * (x.numel() + w.numel() + b.numel() + y.numel())
+        gm, gn, gk = n_ * hw_ * hw_, k_, c_ * 9
+
+        lc = conv.conv2d_forward_kernel.prepare(y, x, w, b, n_, c_, hw_, hw_, k_, hw_, hw_, 3, 3, 1, 1, 1, 1, 1, 1, gm, gn, gk, **cfg)
+        r = measure("CONV", lambda i: lc(), flops, bytes_, "bf16", "mfma")
+        r["tile"] = cfg
+        r["workload"] = "conv2d forward bf16: input [32,256,56,56], weight [256,256,3,3], bias, stride 1, padding 1"
+        ref = oracle.reference_conv2d(x_cpu[5:6], w_cpu, b_cpu, (1, 1), (1, 1), (1, 1))
+        r["parity_ok"] = bool(oracle.within_tolerance(y[5:6], ref)[0])
+        if not args.no_vendor:
+            r["vendor_ms"] = vendor_ms(lambda i: torch_conv2d_forward(x, w, b, (1, 1), (1, 1), (1, 1)))
+            r["vendor_note"] = "torch.nn.functional.conv2d (MIOpen), same tensors"
+        if not args.no_cpu:
+            xf, wf, bf = x_cpu[:2].float(), w_cpu.float(), b_cpu.float()
+            t, n = cpu_time(lambda: torch.nn.functional.conv2d(xf, wf, bf, (1, 1), (1, 1)))
+            r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(flops * 2 / n_ / t / 1e9, 1), "cores": torch.get_num_threads(),
+                        "sample": f"torch fp32 CPU conv2d, first 2 of {n_} images, median of {n}"}
+        del x, w, b, y
 
     # C5: int8 -> int32
     if "C5" in wanted:

@@ -17,7 +17,10 @@
  *     tritonix/ops/swiglu.py:24-110 (phase 1 of swiglu_kernel :155-205);
  *   - the int8 -> int32 kernel playground/test_int8_mma.py:7-42;
  *   - `triton.OutOfResources` as raised by the Triton launcher and caught at
- *     tritonix/autotune.py:134 (here: TNX_E_LDS + tnx_gemm_lds_bytes()).
+ *     tritonix/autotune.py:134 (here: TNX_E_LDS + tnx_gemm_lds_bytes());
+ *   - `conv2d_forward_kernel[grid](output, input, weight, bias, 9 sizes, 6 stride/pad/dilation values,
+ *     GEMM_M, GEMM_N, GEMM_K, BLOCK_SIZE_M=, BLOCK_SIZE_N=, BLOCK_SIZE_K=, GROUP_SIZE_M=, OUT_DTYPE=,
+ *     USE_TF32=)` tritonix/ops/conv2d/forward.py:19-165, launched from :202-311 (tnx_conv2d_forward).
  */
 #ifndef TRITONIX_HIP_H
 #define TRITONIX_HIP_H
@@ -181,6 +184,47 @@ const char* tnx_kernel_name(int i);
  * multiply-add count x 2.  Asynchronous on `stream`; timing is the caller's. */
 int tnx_probe_mfma(int dtype, int mfma_rows, int zero_operands, int workgroups, int iterations, void* scratch,
                    size_t scratch_bytes, void* stream, double* ops_per_launch);
+
+/* ---- conv2d forward (implicit GEMM on the same LDS layout and MFMA fragments) ------------------------------
+ * Stands in for conv2d_forward_kernel, tritonix/ops/conv2d/forward.py:19-165: contiguous NCHW input, KCRS
+ * weight, NCHW output of the input's type, GEMM_M = batch * h_out * w_out, GEMM_N = c_out, GEMM_K = c_in *
+ * filter_h * filter_w, zero padding, fp32 accumulation, optional bias added in fp32 before the one rounding.
+ * block_pixels / block_cout / block_k / group_pixels are the reference's BLOCK_SIZE_M / BLOCK_SIZE_N /
+ * BLOCK_SIZE_K / GROUP_SIZE_M.  dtype is TNX_F16 or TNX_BF16 (the reference's float32-with-TF32 mode has no
+ * matrix instruction on gfx950 and is not built: TNX_E_UNSUPPORTED).  Limits: batch * h_out * w_out and the
+ * element counts of input and weight below 2^31, h_in / w_in / pad / (filter - 1) * dilation at most 16384. */
+typedef struct tnx_conv2d_args {
+  const void* input;   /* [batch, c_in, h_in, w_in]                                 */
+  const void* weight;  /* [c_out, c_in, filter_h, filter_w]                         */
+  const void* bias;    /* [c_out] of bias_dtype, or NULL                            */
+  void* output;        /* [batch, c_out, h_out, w_out], same type as the input      */
+  int32_t batch, c_in, h_in, w_in;
+  int32_t c_out, filter_h, filter_w;
+  int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  int32_t dtype;       /* tnx_dtype of input, weight and output                     */
+  int32_t bias_dtype;  /* TNX_F16 / TNX_BF16 / TNX_F32                              */
+  int32_t block_pixels, block_cout, block_k; /* workgroup tile; 0 0 0 = built-in choice */
+  int32_t group_pixels; /* pixel tiles per L2 group (tl.swizzle2d size_g); 0 = 8    */
+  void* stream;        /* hipStream_t; NULL = the null stream                       */
+} tnx_conv2d_args;
+
+/* Launch one conv2d forward.  Returns a tnx_status.  Asynchronous, allocates nothing. */
+int tnx_conv2d_forward(const tnx_conv2d_args* args);
+
+/* TNX_OK if tnx_conv2d_forward would accept these args (pointers are not inspected, apart from their
+ * alignment), otherwise the status it would return.  Pure host arithmetic. */
+int tnx_conv2d_supported(const tnx_conv2d_args* args);
+
+/* h_out / w_out as the reference computes them (tritonix/ops/conv2d/forward.py:226-227); either may come
+ * back <= 0 for a filter larger than the padded image, which tnx_conv2d_forward rejects. */
+void tnx_conv2d_output_size(const tnx_conv2d_args* args, int32_t* h_out, int32_t* w_out);
+
+/* Fill block_pixels / block_cout / block_k / group_pixels with the built-in choice for this problem. */
+int tnx_conv2d_default_config(tnx_conv2d_args* args);
+
+/* Compiled conv2d tiles: count, and "dtype block_cout block_pixels block_k" of the i-th (static storage). */
+int tnx_conv2d_kernel_count(void);
+const char* tnx_conv2d_kernel_name(int i);
 
 const char* tnx_strerror(int status);
 int tnx_last_hip_error(void); /* hipError_t of the last TNX_E_HIP on this thread */

@@ -27,6 +27,14 @@ product of two plain GEMMs, and the interleave convention; ``reference_*`` are
 library routines.  The reference's own tests hold stored vectors for none of
 these except the trie (tests/test_trie.py), which tests/test_trie.py here
 re-checks.  Split-K, GLU and int8 have no test in the reference at all.
+
+``tiled_conv2d`` (conv_oracle.c) restates conv2d_forward_kernel
+(tritonix/ops/conv2d/forward.py:19-165); the reference holds no test or stored
+vector for it, so tests/test_conv2d_oracle.py pins it against
+``torch.nn.functional.conv2d`` in float64 over asymmetric strides, paddings and
+dilations and against closed forms (1x1 filter = matrix product, one-hot filter
+= shifted copy, all-ones filter = box sums); ``reference_conv2d`` is that library
+routine in fp32.
 """
 from __future__ import annotations
 
@@ -144,9 +152,45 @@ def tiled_glu(x, w12, activation="silu", block_m=32, block_n=32, block_k=16, gro
     return z
 
 
+def conv2d_output_size(h_in, w_in, fh, fw, stride, padding, dilation):
+    ho, wo = ctypes.c_int(), ctypes.c_int()
+    lib().oracle_conv2d_output_size(int(h_in), int(w_in), int(fh), int(fw), int(stride[0]), int(stride[1]), int(padding[0]),
+                                    int(padding[1]), int(dilation[0]), int(dilation[1]), ctypes.byref(ho), ctypes.byref(wo))
+    return ho.value, wo.value
+
+
+def tiled_conv2d(x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1), block_m=32, block_n=32, block_k=16):
+    """conv_oracle.c on float32 numpy arrays: x [N, C, H, W], w [K, C, R, S], bias [K] or None -> y [N, K, HO, WO] fp32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    n, c, h, wd = x.shape
+    k, c2, r, s = w.shape
+    assert c == c2
+    ho, wo = conv2d_output_size(h, wd, r, s, stride, padding, dilation)
+    assert ho > 0 and wo > 0, "empty output"
+    y = np.empty((n, k, ho, wo), dtype=np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    f = lib().oracle_conv2d_f32
+    f.restype = ctypes.c_int
+    rc = f(_fp(x), _fp(w), None if b is None else _fp(b), _fp(y), n, c, h, wd, k, r, s, int(stride[0]), int(stride[1]),
+           int(padding[0]), int(padding[1]), int(dilation[0]), int(dilation[1]), int(block_m), int(block_n), int(block_k))
+    assert rc == 0, rc
+    return y
+
+
 # ---------------------------------------------------------------------------
 # what the reference checks against: torch CPU, fp32 (exact int32 for int8)
 # ---------------------------------------------------------------------------
+def reference_conv2d(x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """``torch.nn.functional.conv2d`` of the upcast inputs in fp32 on the CPU: the reference's own baseline
+    (torch_conv2d_forward, tritonix/ops/conv2d/forward.py:314-323)."""
+    import torch
+
+    b = None if bias is None else bias.detach().cpu().float()
+    return torch.nn.functional.conv2d(x.detach().cpu().float(), w.detach().cpu().float(), b, stride, padding, dilation)
+
+
+
 def reference_matmul(a, b):
     """fp32 CPU matmul of the upcast inputs; int8 inputs give the exact int32 product (via float64)."""
     import torch

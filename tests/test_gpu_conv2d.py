@@ -1,0 +1,175 @@
+"""conv2d forward on the GPU against the CPU oracle (tritonix/ops/conv2d/forward.py:19-165, :202-311).
+
+Tolerance: the kernel accumulates in fp32 and rounds once to the 16-bit output type, the oracle keeps fp32; the
+bar is the one of the GEMM tests, |out - ref| <= 1e-2 * (|ref| + rms(ref)).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tritonix_amd import _C
+from tritonix_amd.ops.conv2d import conv2d_forward, conv2d_forward_kernel, torch_conv2d_forward
+from tritonix_amd.ops.conv2d import forward as conv
+
+pytestmark = pytest.mark.gpu
+
+CASES = {
+    # n, c_in, h, w, c_out, r, s, stride, padding, dilation, bias
+    "3x3_same": (2, 16, 16, 16, 32, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    "1x1_flat": (1, 8, 8, 8, 16, 1, 1, (1, 1), (0, 0), (1, 1), False),
+    "7x7_stem_ragged_k": (3, 3, 19, 23, 20, 7, 7, (2, 2), (3, 3), (1, 1), True),
+    "w_out_14": (2, 24, 14, 14, 40, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    "all_asymmetric": (2, 16, 17, 13, 24, 3, 2, (1, 2), (2, 0), (2, 1), False),
+    "1x1_stride2": (2, 32, 28, 28, 64, 1, 1, (2, 2), (0, 0), (1, 1), False),
+    "one_pixel": (1, 5, 5, 5, 7, 5, 5, (1, 1), (0, 0), (1, 1), True),
+    "dilated_wide_pad": (2, 32, 9, 9, 200, 3, 3, (1, 1), (2, 2), (2, 2), True),
+    "odd_plane_7x7": (3, 16, 7, 7, 24, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    "pad_wider_than_filter": (1, 8, 6, 6, 8, 3, 3, (1, 1), (4, 4), (1, 1), False),
+    "tiny_tensor": (1, 1, 2, 3, 2, 1, 1, (1, 1), (0, 0), (1, 1), True),
+}
+TILES = [(64, 64, 32), (128, 128, 64), (64, 128, 64), (128, 64, 32), (256, 128, 64), (128, 256, 64)]   # BLOCK_SIZE_M, _N, _K
+
+
+def _inputs(case, dtype, seed=0):
+    n, c, h, w, k, r, s, stride, padding, dilation, has_bias = case
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, c, h, w, generator=g).to(dtype)
+    wt = (torch.randn(k, c, r, s, generator=g) / (c * r * s) ** 0.5).to(dtype)
+    b = torch.randn(k, generator=g).to(dtype) if has_bias else None
+    return x, wt, b, stride, padding, dilation
+
+
+def _oracle(x, wt, b, stride, padding, dilation):
+    y = oracle.tiled_conv2d(x.float().numpy(), wt.float().numpy(), None if b is None else b.float().numpy(), stride, padding,
+                            dilation, 32, 32, 16)
+    return torch.from_numpy(y)
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_conv2d_matches_the_oracle(name, dtype, device):
+    x, wt, b, stride, padding, dilation = _inputs(CASES[name], dtype, seed=len(name))
+    ref = _oracle(x, wt, b, stride, padding, dilation)
+    for bm, bn, bk in TILES:
+        cfg = dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=4)
+        out = conv2d_forward(x.to(device), wt.to(device), None if b is None else b.to(device), stride, padding, dilation,
+                             config=cfg)
+        assert out.dtype == dtype and tuple(out.shape) == tuple(ref.shape)
+        ok, err, rel = oracle.within_tolerance(out, ref)
+        assert ok, (name, dtype, cfg, err, rel)
+
+
+def test_float32_bias_and_no_bias_agree_with_the_oracle(device):
+    x, wt, _, stride, padding, dilation = _inputs(CASES["3x3_same"], torch.bfloat16, seed=3)
+    b32 = torch.randn(wt.shape[0], generator=torch.Generator().manual_seed(4))
+    out = conv2d_forward(x.to(device), wt.to(device), b32.to(device), stride, padding, dilation,
+                         config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64))
+    assert oracle.within_tolerance(out, _oracle(x, wt, b32, stride, padding, dilation))[0]
+
+
+def test_tiles_agree_bit_for_bit_when_k_order_is_the_same(device):
+    """Two tiles with the same block_k add the same products in the same order: their outputs are identical."""
+    x, wt, b, stride, padding, dilation = _inputs(CASES["w_out_14"], torch.bfloat16, seed=7)
+    outs = [conv2d_forward(x.to(device), wt.to(device), b.to(device), stride, padding, dilation,
+                           config=dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=64))
+            for bm, bn in ((64, 64), (128, 128), (64, 128), (128, 64))]
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
+def test_one_by_one_filter_equals_the_gemm_engine(device):
+    """A 1x1, stride-1 conv is W[c_out, c_in] @ X[c_in, pixels] per image: the conv kernel and the GEMM kernel
+    must round the same fp32 sums (same block_k, same accumulation order along k)."""
+    import tritonix_amd
+
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, 64, 16, 16, generator=g).bfloat16().to(device)
+    wt = (torch.randn(128, 64, 1, 1, generator=g) / 8).bfloat16().to(device)
+    out = conv2d_forward(x, wt, None, config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64))
+    for img in range(2):
+        with tritonix_amd.matmul.force_backend("triton"):
+            want = tritonix_amd.matmul(wt.view(128, 64), x[img].reshape(64, 256))
+        assert oracle.within_tolerance(out[img].reshape(128, 256), want.float().cpu(), rel=4e-3)[0]
+
+
+def test_mini_tuner_picks_a_candidate_and_remembers_it(device):
+    conv._CONV_FWD_CONFIG_CACHE.clear()
+    x, wt, b, stride, padding, dilation = _inputs(CASES["w_out_14"], torch.float16, seed=5)
+    out = conv2d_forward(x.to(device), wt.to(device), b.to(device), stride, padding, dilation)
+    assert len(conv._CONV_FWD_CONFIG_CACHE) == 1
+    (key, cfg), = conv._CONV_FWD_CONFIG_CACHE.items()
+    assert key[-1] == torch.float16 and set(cfg) == {"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "GROUP_SIZE_M"}
+    assert oracle.within_tolerance(out, _oracle(x, wt, b, stride, padding, dilation))[0]
+    again = conv2d_forward(x.to(device), wt.to(device), b.to(device), stride, padding, dilation)
+    assert torch.equal(out, again) and len(conv._CONV_FWD_CONFIG_CACHE) == 1
+
+
+def test_kernel_launch_object_with_the_reference_arguments(device):
+    x, wt, b, stride, padding, dilation = _inputs(CASES["all_asymmetric"], torch.bfloat16, seed=9)
+    n, c, h, w = x.shape
+    k, _, r, s = wt.shape
+    ho, wo = conv.output_size(h, w, r, s, stride, padding, dilation)
+    xd, wd = x.to(device), wt.to(device)
+    out = torch.empty(n, k, ho, wo, dtype=x.dtype, device=device)
+    grid = (conv.cdiv(n * ho * wo, 64), conv.cdiv(k, 64))
+    conv2d_forward_kernel[grid](out, xd, wd, None, n, c, h, w, k, ho, wo, r, s, stride[0], stride[1], padding[0], padding[1],
+                                dilation[0], dilation[1], n * ho * wo, k, c * r * s, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64,
+                                BLOCK_SIZE_K=32, GROUP_SIZE_M=8, USE_TF32=True)
+    assert oracle.within_tolerance(out, _oracle(x, wt, None, stride, padding, dilation))[0]
+
+
+def test_through_the_c_abi_with_the_built_in_tile(device):
+    import ctypes
+
+    x, wt, b, stride, padding, dilation = _inputs(CASES["dilated_wide_pad"], torch.float16, seed=13)
+    xd, wd, bd = x.to(device), wt.to(device), b.to(device)
+    ref = _oracle(x, wt, b, stride, padding, dilation)
+    out = torch.empty(ref.shape, dtype=x.dtype, device=device)
+    a = _C.Conv2dArgs()
+    a.input, a.weight, a.bias, a.output = xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), out.data_ptr()
+    a.batch, a.c_in, a.h_in, a.w_in = x.shape
+    a.c_out, _, a.filter_h, a.filter_w = wt.shape
+    (a.stride_h, a.stride_w), (a.pad_h, a.pad_w), (a.dil_h, a.dil_w) = stride, padding, dilation
+    a.dtype = a.bias_dtype = _C.F16
+    a.stream = torch.cuda.current_stream().cuda_stream
+    assert _C.load().tnx_conv2d_forward(ctypes.byref(a)) == _C.OK        # block_* == 0: built-in choice
+    torch.cuda.synchronize()
+    assert oracle.within_tolerance(out, ref)[0]
+
+
+def test_resnet_layer_at_size_against_the_vendor_routine_and_linearity(device):
+    """Batch 32, 256 -> 256 channels, 56x56, 3x3: too large for the CPU oracle, so the checks are (i) sampled output
+    planes against the oracle's fp32 library routine on the CPU, (ii) the vendor's GPU conv2d within the rounding
+    of two bf16 results, (iii) conv(x, w1) + conv(x, w2) == conv(x, w1 + w2) when w1, w2 have disjoint support."""
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(32, 256, 56, 56, generator=g).bfloat16()
+    wt = (torch.randn(256, 256, 3, 3, generator=g) / 48).bfloat16()
+    b = torch.randn(256, generator=g).bfloat16()
+    xd, wd, bd = x.to(device), wt.to(device), b.to(device)
+    out = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1))
+    for img in (0, 17, 31):
+        ref = oracle.reference_conv2d(x[img:img + 1], wt, b, (1, 1), (1, 1), (1, 1))
+        assert oracle.within_tolerance(out[img:img + 1], ref)[0]
+    vendor = torch_conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1))
+    assert oracle.within_tolerance(out, vendor.float().cpu(), rel=2e-2)[0]
+    mask = torch.zeros_like(wd)
+    mask[:, :128] = 1
+    y1 = conv2d_forward(xd, wd * mask, None, (1, 1), (1, 1), (1, 1)).float()
+    y2 = conv2d_forward(xd, wd * (1 - mask), None, (1, 1), (1, 1), (1, 1)).float()
+    y = conv2d_forward(xd, wd, None, (1, 1), (1, 1), (1, 1)).float()
+    assert oracle.within_tolerance((y1 + y2).cpu(), y.cpu(), rel=2e-2)[0]
+
+
+def test_zero_input_and_identity_filter(device):
+    x = torch.zeros(2, 8, 9, 9, dtype=torch.bfloat16, device=device)
+    wt = torch.randn(16, 8, 3, 3, device=device).bfloat16()
+    b = torch.randn(16, device=device).bfloat16()
+    out = conv2d_forward(x, wt, b, (1, 1), (1, 1), (1, 1), config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=32))
+    assert torch.equal(out, b.view(1, 16, 1, 1).expand_as(out))
+    # centre tap = identity matrix: the output is the input, bit for bit
+    x = torch.randn(2, 16, 10, 12, device=device).bfloat16()
+    wt = torch.zeros(16, 16, 3, 3, dtype=torch.bfloat16, device=device)
+    wt[torch.arange(16), torch.arange(16), 1, 1] = 1
+    out = conv2d_forward(x, wt, None, (1, 1), (1, 1), (1, 1), config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64))
+    assert torch.equal(out, x)

@@ -24,12 +24,24 @@ def test_reference_import_lines_work():
     assert isinstance(matmul_kernel, TunableKernel)
 
 
+def test_conv2d_forward_import_lines_work():
+    import tritonix
+    import tritonix_amd
+    from tritonix.ops.conv2d import conv2d_forward, conv2d_forward_kernel, torch_conv2d_forward   # noqa: F401
+    from tritonix.ops.conv2d.forward import conv2d_forward as same
+
+    assert tritonix.conv2d_forward is tritonix_amd.conv2d_forward is conv2d_forward is same
+    assert tritonix.torch_conv2d_forward is torch_conv2d_forward
+
+
 def test_operators_off_the_path_are_absent():
     with pytest.raises(ImportError):
-        import tritonix.ops.conv2d                                                            # noqa: F401
+        import tritonix.ops.statistics                                                        # noqa: F401
+    with pytest.raises(ImportError):
+        import tritonix.ops.conv2d.backward                                                   # noqa: F401
     import tritonix
 
-    assert not hasattr(tritonix, "conv2d_forward") and not hasattr(tritonix, "topk")
+    assert not hasattr(tritonix, "topk") and not hasattr(tritonix, "conv2d_grad_input_kernel")
 
 
 def test_forced_oracle_backend_through_the_alias():

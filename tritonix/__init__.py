@@ -6,16 +6,17 @@ examples/tune_matmul.py:1-10 of the reference).  This package maps those module 
 ``tritonix_amd`` so such code runs unchanged on the HIP kernels: every ``tritonix.x.y`` below *is* the module
 ``tritonix_amd.x.y`` (one module object, two names), nothing is re-implemented here.
 
-Only the dense tiled-GEMM path exists: ``tritonix.ops.conv2d``, ``tritonix.ops.statistics`` and the other
-operators of the reference are not provided and importing them raises ``ImportError``.
+Only the dense tiled-GEMM path and conv2d forward exist: ``tritonix.ops.conv2d.backward``,
+``tritonix.ops.statistics`` and the other operators of the reference are not provided and importing them raises
+``ImportError``.
 """
 import importlib
 import sys
 
 import tritonix_amd
 
-_ALIASED = ("autotune", "dispatcher", "testing", "kernel", "ops", "ops.matmul", "ops.swiglu", "utils", "utils.spaces",
-            "utils.pruners")
+_ALIASED = ("autotune", "dispatcher", "testing", "kernel", "ops", "ops.matmul", "ops.swiglu", "ops.conv2d",
+            "ops.conv2d.forward", "utils", "utils.spaces", "utils.pruners")
 
 for _name in _ALIASED:
     sys.modules[f"{__name__}.{_name}"] = importlib.import_module(f"tritonix_amd.{_name}")

@@ -28,7 +28,8 @@ STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
            "tnx_gemm_default_config", "tnx_tile_coords", "tnx_probe_mfma", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
-           "tnx_last_hip_error", "tnx_version")
+           "tnx_last_hip_error", "tnx_version", "tnx_conv2d_forward", "tnx_conv2d_supported", "tnx_conv2d_output_size",
+           "tnx_conv2d_default_config", "tnx_conv2d_kernel_count", "tnx_conv2d_kernel_name")
 
 
 class GemmArgs(ctypes.Structure):
@@ -45,6 +46,21 @@ class GemmArgs(ctypes.Structure):
         ("num_stages", ctypes.c_int32), ("num_warps", ctypes.c_int32),
         ("epilogue", ctypes.c_int32), ("tail_tiles", ctypes.c_int32), ("schedule", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+class Conv2dArgs(ctypes.Structure):
+    """struct tnx_conv2d_args"""
+    _fields_ = [
+        ("input", ctypes.c_void_p), ("weight", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("output", ctypes.c_void_p),
+        ("batch", ctypes.c_int32), ("c_in", ctypes.c_int32), ("h_in", ctypes.c_int32), ("w_in", ctypes.c_int32),
+        ("c_out", ctypes.c_int32), ("filter_h", ctypes.c_int32), ("filter_w", ctypes.c_int32),
+        ("stride_h", ctypes.c_int32), ("stride_w", ctypes.c_int32), ("pad_h", ctypes.c_int32), ("pad_w", ctypes.c_int32),
+        ("dil_h", ctypes.c_int32), ("dil_w", ctypes.c_int32),
+        ("dtype", ctypes.c_int32), ("bias_dtype", ctypes.c_int32),
+        ("block_pixels", ctypes.c_int32), ("block_cout", ctypes.c_int32), ("block_k", ctypes.c_int32),
+        ("group_pixels", ctypes.c_int32),
         ("stream", ctypes.c_void_p),
     ]
 
@@ -89,6 +105,16 @@ def load() -> ctypes.CDLL:
     lib.tnx_last_hip_error.restype = ctypes.c_int
     lib.tnx_version.argtypes = []
     lib.tnx_version.restype = ctypes.c_int
+    cp = ctypes.POINTER(Conv2dArgs)
+    for name in ("tnx_conv2d_forward", "tnx_conv2d_supported", "tnx_conv2d_default_config"):
+        getattr(lib, name).argtypes = [cp]
+        getattr(lib, name).restype = ctypes.c_int
+    lib.tnx_conv2d_output_size.argtypes = [cp, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
+    lib.tnx_conv2d_output_size.restype = None
+    lib.tnx_conv2d_kernel_count.argtypes = []
+    lib.tnx_conv2d_kernel_count.restype = ctypes.c_int
+    lib.tnx_conv2d_kernel_name.argtypes = [ctypes.c_int]
+    lib.tnx_conv2d_kernel_name.restype = ctypes.c_char_p
     _lib = lib
     return lib
 
@@ -122,6 +148,11 @@ def tile_coords(schedule: int, idx: int, tiles_m: int, tiles_n: int, group_m: in
     if status != OK:
         raise ValueError(strerror(status))
     return tm.value, tn.value
+
+
+def conv2d_kernel_names():
+    lib = load()
+    return [lib.tnx_conv2d_kernel_name(i).decode() for i in range(lib.tnx_conv2d_kernel_count())]
 
 
 def kernel_names():

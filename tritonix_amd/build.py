@@ -100,6 +100,36 @@ def instance_list(quick=False):
     return out
 
 
+def conv_instance_list(quick=False):
+    """(dtype, block_cout, block_pixels, block_k) of every conv2d forward tile to build (four waves, two LDS slots).
+
+    The reference's own candidates (tritonix/ops/conv2d/forward.py:172-180: pixels x channels in {64, 128}^2,
+    block_k in {32, 64}) and two larger tiles."""
+    out = []
+    for dt in ("bf16", "f16"):
+        for bc, bp in ((64, 64), (64, 128), (128, 64), (128, 128), (256, 128), (128, 256)):
+            for bk in (32, 64):
+                if max(bc, bp) == 256 and bk == 32:
+                    continue
+                if quick and not ((bc, bp) in ((128, 128), (64, 64)) and bk == 64):
+                    continue
+                assert tile_valid(2, bc, bp, bk, 4, 2)
+                out.append((dt, bc, bp, bk))
+    return out
+
+
+def parse_only_conv(spec):
+    """'bf16:128:128:64,...' (dtype:block_cout:block_pixels:block_k) for development builds."""
+    out = []
+    for item in spec.split(","):
+        dt, *nums = item.strip().split(":")
+        bc, bp, bk = (int(v) for v in nums)
+        if dt not in ("bf16", "f16") or not tile_valid(2, bc, bp, bk, 4, 2):
+            raise SystemExit(f"{item}: not a buildable conv2d tile")
+        out.append((dt, bc, bp, bk))
+    return out
+
+
 def write_if_changed(path, text):
     if os.path.exists(path):
         with open(path) as f:
@@ -107,6 +137,37 @@ def write_if_changed(path, text):
                 return
     with open(path, "w") as f:
         f.write(text)
+
+
+def generate_conv(instances, gen):
+    """Instance files of the conv2d tiles, one per (dtype, block_cout), and their table."""
+    groups = {}
+    for inst in instances:
+        groups.setdefault((inst[0], inst[1]), []).append(inst)
+    files, names = [], []
+    for (dt, bc), items in sorted(groups.items()):
+        name = f"conv_{dt}_c{bc}"
+        tag = TAGS[dt][0]
+        rows = ",\n".join(f"    TNX_CONV_ENTRY({tag}, {i[1]}, {i[2]}, {i[3]})" for i in items)
+        text = (f'// generated by tritonix_amd/build.py -- do not edit\n#include "{CSRC}/conv_tile.h"\n'
+                f"namespace tnx {{\nstatic ConvEntry k_{name}[] = {{\n{rows}\n}};\n"
+                f"ConvGroup g_{name} = {{k_{name}, {len(items)}}};\n}}\n")
+        path = os.path.join(gen, name + ".hip")
+        write_if_changed(path, text)
+        files.append(path)
+        names.append(name)
+    decl = "\n".join(f"extern ConvGroup g_{n};" for n in names)
+    arr = ", ".join(f"g_{n}" for n in names)
+    n = len(names)
+    body = (f"  static ConvGroup all[{max(n, 1)}];\n  static bool init = false;\n"
+            f"  if (!init) {{ {'ConvGroup tmp[] = {' + arr + '}; for (int i = 0; i < ' + str(n) + '; ++i) all[i] = tmp[i]; ' if n else ''}init = true; }}\n")
+    text = (f'// generated by tritonix_amd/build.py -- do not edit\n#include "{CSRC}/conv_tile.h"\nnamespace tnx {{\n{decl}\n}}\n'
+            f"using namespace tnx;\n"
+            f'extern "C" const ConvGroup* tnx_conv_groups(int* n) {{\n{body}  *n = {n};\n  return all;\n}}\n')
+    path = os.path.join(gen, "conv_groups.hip")
+    write_if_changed(path, text)
+    files.append(path)
+    return files
 
 
 def generate(instances):
@@ -130,10 +191,13 @@ def generate(instances):
         names.append(name)
     decl = "\n".join(f"extern KernelGroup g_{n};" for n in names)
     arr = ", ".join(f"g_{n}" for n in names)
+    n = len(names)
+    fill = f"KernelGroup tmp[] = {{{arr}}}; for (int i = 0; i < {n}; ++i) all[i] = tmp[i]; " if n else ""
     text = (f'// generated by tritonix_amd/build.py -- do not edit\n#include "{CSRC}/registry.h"\nnamespace tnx {{\n{decl}\n}}\n'
             f"using namespace tnx;\n"
             f'extern "C" const KernelGroup* tnx_kernel_groups(int* n) {{\n'
-            f"  static KernelGroup all[{len(names)}];\n  static bool init = false;\n  if (!init) {{ KernelGroup tmp[] = {{{arr}}}; for (int i = 0; i < {len(names)}; ++i) all[i] = tmp[i]; init = true; }}\n  *n = {len(names)};\n  return all;\n}}\n")
+            f"  static KernelGroup all[{max(n, 1)}];\n  static bool init = false;\n  if (!init) {{ {fill}init = true; }}\n"
+            f"  *n = {n};\n  return all;\n}}\n")
     path = os.path.join(gen, "groups.hip")
     write_if_changed(path, text)
     files.append(path)
@@ -142,6 +206,7 @@ def generate(instances):
 
 def _compile(src, obj, verbose, force=True):
     deps = [src, os.path.join(CSRC, "gemm_tile.h"), os.path.join(CSRC, "gemm_skinny.h"), os.path.join(CSRC, "registry.h"),
+            os.path.join(CSRC, "conv_tile.h"),
             os.path.join(ROOT, "include", "tritonix_hip.h"), os.path.abspath(__file__)]
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(d) for d in deps):
         return obj
@@ -155,25 +220,28 @@ def _compile(src, obj, verbose, force=True):
     return obj
 
 
-def build(jobs=None, quick=False, verbose=True, force=True, only=None, out=None, defines=()):
+def build(jobs=None, quick=False, verbose=True, force=True, only=None, out=None, defines=(), only_conv=None):
     """Compile every kernel for gfx950 and link the shared library.
 
     ``only`` / ``out`` / ``defines`` are for development builds: a few tiles, linked to another path, with extra
     ``-D`` macros; they use their own object directory so the full build's objects stay valid."""
     global BUILD
     jobs = jobs or min(8, os.cpu_count() or 1)
-    instances = parse_only(only) if only else instance_list(quick=quick)
+    instances = parse_only(only) if only else ([] if only_conv else instance_list(quick=quick))
+    conv_instances = parse_only_conv(only_conv) if only_conv else ([] if only else conv_instance_list(quick=quick))
     lib = out or LIB
-    if only or out or defines:
+    if only or only_conv or out or defines:
         BUILD = os.path.join(ROOT, "build", "dev_" + os.path.basename(lib).replace(".", "_"))
     DEVICE_FLAGS.extend(f"-D{d}" for d in defines)
-    srcs = generate(instances) + [os.path.join(CSRC, "capi.hip"), os.path.join(CSRC, "skinny.hip"),
-                                  os.path.join(CSRC, "probe.hip")]
+    srcs = generate(instances) + generate_conv(conv_instances, os.path.join(BUILD, "gen")) + [
+        os.path.join(CSRC, "capi.hip"), os.path.join(CSRC, "skinny.hip"), os.path.join(CSRC, "probe.hip"),
+        os.path.join(CSRC, "conv.hip")]
     objdir = os.path.join(BUILD, "obj")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in srcs]
     if verbose:
-        print(f"building {len(instances)} tile kernels in {len(srcs)} translation units, {jobs} jobs", flush=True)
+        print(f"building {len(instances)} GEMM and {len(conv_instances)} conv2d tile kernels in {len(srcs)} translation units, "
+              f"{jobs} jobs", flush=True)
     t0 = time.time()
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda so: _compile(so[0], so[1], verbose, force), zip(srcs, objs)))
@@ -194,10 +262,12 @@ def main(argv=None):
     ap.add_argument("--quick", action="store_true", help="build a small subset of the tile kernels (development)")
     ap.add_argument("--incremental", action="store_true", help="development: keep objects that are newer than their sources")
     ap.add_argument("--only", default=None, help="development: build just these tiles, dtype:bm:bn:bk:warps:stages,...")
+    ap.add_argument("--only-conv", default=None, help="development: build just these conv2d tiles, dtype:cout:pixels:bk,...")
     ap.add_argument("--out", default=None, help="development: link to this path instead of the package's library")
     ap.add_argument("-D", dest="defines", action="append", default=[], help="development: extra macro for the device code")
     args = ap.parse_args(argv)
-    build(jobs=args.jobs, quick=args.quick, only=args.only, out=args.out, defines=args.defines, force=not args.incremental)
+    build(jobs=args.jobs, quick=args.quick, only=args.only, out=args.out, defines=args.defines, force=not args.incremental,
+          only_conv=args.only_conv)
     return 0
 
 

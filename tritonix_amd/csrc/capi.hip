@@ -14,6 +14,9 @@ using namespace tnx;
 extern "C" const KernelGroup* tnx_kernel_groups(int* ngroups);  // generated
 
 static thread_local int g_last_hip_error = 0;
+namespace tnx {
+void note_hip_error(int err) { g_last_hip_error = err; }
+}
 
 static int elem_size(int dt) { return dt == TNX_I8 ? 1 : (dt == TNX_F16 || dt == TNX_BF16) ? 2 : 4; }
 

@@ -18,6 +18,9 @@ struct KernelEntry {
   launch_fn fast_bt;  // DMA loader for k-contiguous B (stride_bk == 1, the `x @ w.t()` layout); may be null
 };
 
+// records the hipError_t behind a TNX_E_HIP for tnx_last_hip_error() (per thread)
+void note_hip_error(int err);
+
 struct KernelGroup {
   KernelEntry* entries;
   int count;
