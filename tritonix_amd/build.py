@@ -104,10 +104,10 @@ def conv_instance_list(quick=False):
     """(dtype, block_cout, block_pixels, block_k) of every conv2d forward tile to build (four waves, two LDS slots).
 
     The reference's own candidates (tritonix/ops/conv2d/forward.py:172-180: pixels x channels in {64, 128}^2,
-    block_k in {32, 64}) and two larger tiles."""
+    block_k in {32, 64}) and three larger tiles."""
     out = []
     for dt in ("bf16", "f16"):
-        for bc, bp in ((64, 64), (64, 128), (128, 64), (128, 128), (256, 128), (128, 256)):
+        for bc, bp in ((64, 64), (64, 128), (128, 64), (128, 128), (256, 64), (256, 128), (128, 256)):
             for bk in (32, 64):
                 if max(bc, bp) == 256 and bk == 32:
                     continue

@@ -106,6 +106,18 @@ static int resolve(const tnx_conv2d_args* a, const ConvEntry** entry, ConvParams
   p->div_w_out = make_fastdiv((uint32_t)w_out);
   p->div_rs = make_fastdiv((uint32_t)(a->filter_h * a->filter_w));
   p->div_s = make_fastdiv((uint32_t)a->filter_w);
+  {
+    // block_k = sc * (R*S) + sh * S + sw
+    const int rs = a->filter_h * a->filter_w;
+    const int sc = bk / rs, sh = (bk % rs) / a->filter_w, sw = bk % a->filter_w;
+    p->step_dw = sw * a->dil_w;
+    p->step_dh = sh * a->dil_h;
+    p->step_koff = sc * p->hw_in + p->step_dh * a->w_in + p->step_dw;
+    p->lim_w = a->filter_w * a->dil_w;
+    p->lim_h = a->filter_h * a->dil_h;
+    p->adj_w = a->dil_h * a->w_in - p->lim_w;          // dw wraps: one filter row down
+    p->adj_h = p->hw_in - p->lim_h * a->w_in;          // dh wraps: next input channel
+  }
   p->tiles_cout = (int)tiles_cout;
   p->tiles_pix = (int)tiles_pix;
   p->group = a->group_pixels > 0 ? a->group_pixels : 8;

@@ -51,6 +51,9 @@ struct ConvParams {
   uint32_t x_bytes, w_bytes;   // sizes of the input and weight tensors
   int x_last_vec;         // batch * c_in * h_in * w_in - 8: last element offset a 16-byte load may start at (negative: none)
   FastDiv div_hw_out, div_w_out, div_rs, div_s;
+  // one K slab further (block_k taps along (c_in, fh, fw)): what is added to a tap's (dw, dh, element offset), the limits
+  // at which dw and dh wrap, and what a wrap adds to the element offset
+  int step_dw, step_dh, step_koff, lim_w, lim_h, adj_w, adj_h;
   int tiles_cout, tiles_pix, group;
   int bias_dtype;
   bool w_vec_ok;          // weight rows take 16-byte loads: gemm_k % 8 == 0 and a 16-byte aligned base
@@ -82,8 +85,11 @@ struct __attribute__((packed, aligned(2))) Loose16 {
 };
 
 // C = TileCfg<T, block_cout, block_pix, block_k, 4 waves, 2 slots>
+#ifndef TNX_CONV_OCC
+#define TNX_CONV_OCC 1
+#endif
 template <class T, class C>
-__global__ __launch_bounds__(C::THREADS) void conv2d_tile_kernel(ConvParams p) {
+__global__ __launch_bounds__(C::THREADS, TNX_CONV_OCC) void conv2d_tile_kernel(ConvParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK;
   constexpr int MI = C::MI, TM = C::TM, TN = C::TN, THREADS = C::THREADS;
   static_assert(C::VALID && ES == 2 && C::STAGES == 2 && MI == 16, "conv2d is built for 16-bit floats, two LDS slots");
@@ -162,39 +168,71 @@ __global__ __launch_bounds__(C::THREADS) void conv2d_tile_kernel(ConvParams p) {
   const __amdgpu_buffer_rsrc_t xwin = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.x), 0, p.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t wwin = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w), 0, p.w_bytes, 0x00020000);
 
+  // Per chunk of this thread, set up once: the weight chunk's byte offset at slab 0, and the im2col chunk's filter
+  // tap (dh, dw) = (tap row * dil_h, tap column * dil_w) with its element offset c_in * plane + dh * w_in + dw.
+  // load_regs is called for slabs 0, 1, 2, ... in order and moves every tap one slab (block_k taps) on after use,
+  // with additions and wrap-arounds only: the integer divisions and multiplications of the k -> (c_in, fh, fw)
+  // decomposition run once per thread, not once per chunk and slab (32-bit multiplies are quarter rate).
+  uint32_t a_off[A_CH];
+  int a_k[A_CH];
+  bool a_ok[A_CH];
+#pragma unroll
+  for (int q = 0; q < A_CH; ++q) {
+    const int P = q * THREADS + tid;
+    const int row = P / C::CPR_A, cs = P % C::CPR_A;
+    a_k[q] = cs * 8;
+    a_ok[q] = m0 + row < p.c_out;
+    a_off[q] = (uint32_t)((m0 + row) * p.gemm_k + cs * 8) * 2u;
+  }
+  int tap_dh[B_CH], tap_dw[B_CH];
+  uint32_t tap_off[B_CH];      // unsigned: past the last k it keeps growing unused and may wrap
+#pragma unroll
+  for (int q = 0; q < B_CH; ++q) {
+    const int gk = q * B_ROWS + b_row0;
+    const int cin = (int)fd_div((uint32_t)gk, p.div_rs);
+    const int r = gk - cin * (p.fh * p.fw);
+    const int tap_h = (int)fd_div((uint32_t)r, p.div_s);
+    const int tap_w = r - tap_h * p.fw;
+    tap_dh[q] = tap_h * p.dil_h;
+    tap_dw[q] = tap_w * p.dil_w;
+    tap_off[q] = (uint32_t)(cin * p.hw_in + tap_dh[q] * p.w_in + tap_dw[q]);
+  }
+
   auto load_regs = [&](int kt) __attribute__((always_inline)) {
     const int k0 = kt * BK;
     // weights
 #pragma unroll
     for (int q = 0; q < A_CH; ++q) {
-      const int P = q * THREADS + tid;
-      const int row = P / C::CPR_A, cs = P % C::CPR_A;
-      const int gm = m0 + row, gk = k0 + cs * 8;
-      const uint32_t off = (uint32_t)(gm * p.gemm_k + gk) * 2u;
+      const int gk = k0 + a_k[q];
+      const uint32_t off = a_off[q] + (uint32_t)k0 * 2u;
       if (p.w_vec_ok) {
-        st_a[q] = __builtin_amdgcn_raw_buffer_load_b128(wwin, gm < p.c_out && gk < p.gemm_k ? off : OUTSIDE, 0, 0);
+        st_a[q] = __builtin_amdgcn_raw_buffer_load_b128(wwin, a_ok[q] && gk < p.gemm_k ? off : OUTSIDE, 0, 0);
       } else {
         // ragged or unaligned rows (c_in * R * S not a multiple of 8): element loads; rare, and allowed to wait
         uint32_t e[8];
 #pragma unroll
         for (int x = 0; x < 8; ++x)
-          e[x] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(wwin, gm < p.c_out && gk + x < p.gemm_k ? off + 2u * x : OUTSIDE, 0, 0);
+          e[x] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(wwin, a_ok[q] && gk + x < p.gemm_k ? off + 2u * x : OUTSIDE, 0, 0);
         st_a[q] = i32x4{(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16)), (int)(e[4] | (e[5] << 16)), (int)(e[6] | (e[7] << 16))};
       }
     }
     // im2col
 #pragma unroll
     for (int q = 0; q < B_CH; ++q) {
-      const int gk = k0 + q * B_ROWS + b_row0;
-      int dh = 1 << 20, dw = 0, koff = 0;      // k past the end: a tap far outside every image
-      if (gk < p.gemm_k) {
-        const int cin = (int)fd_div((uint32_t)gk, p.div_rs);
-        const int r = gk - cin * (p.fh * p.fw);
-        const int tap_h = (int)fd_div((uint32_t)r, p.div_s);
-        const int tap_w = r - tap_h * p.fw;
-        dh = tap_h * p.dil_h;
-        dw = tap_w * p.dil_w;
-        koff = cin * p.hw_in + dh * p.w_in + dw;
+      // this chunk's tap, then one slab further for the next call (no multiply, no divide: see the set-up below)
+      const bool k_ok = k0 + q * B_ROWS + b_row0 < p.gemm_k;
+      const int dh = k_ok ? tap_dh[q] : 1 << 20;      // k past the end: a tap far outside every image
+      const int dw = tap_dw[q], koff = k_ok ? (int)tap_off[q] : 0;
+      {
+        int ndw = tap_dw[q] + p.step_dw;
+        const bool wrap_w = ndw >= p.lim_w;
+        ndw -= wrap_w ? p.lim_w : 0;
+        int ndh = tap_dh[q] + p.step_dh + (wrap_w ? p.dil_h : 0);
+        const bool wrap_h = ndh >= p.lim_h;
+        ndh -= wrap_h ? p.lim_h : 0;
+        tap_off[q] += (uint32_t)(p.step_koff + (wrap_w ? p.adj_w : 0) + (wrap_h ? p.adj_h : 0));
+        tap_dw[q] = ndw;
+        tap_dh[q] = ndh;
       }
       const int h0 = col_hw[0] >> 16, w0 = (int)(int16_t)(col_hw[0] & 0xffff);
       const int o = col_off[0] + koff;
@@ -237,12 +275,15 @@ __global__ __launch_bounds__(C::THREADS) void conv2d_tile_kernel(ConvParams p) {
         const int lo = (int)(st_m[q] & 0xff), hi = (int)(st_m[q] >> 8);
         v = i32x4{(int)st_b[q][0], (int)st_b[q][1], (int)st_b[q][2], (int)st_b[q][3]};
         if (hi - lo < 8) {
+          // element e stays when lo <= e < hi: two packed 16-bit subtractions whose sign bits, spread by an arithmetic
+          // shift, are the two halves of the test
+          typedef short s16x2 __attribute__((ext_vector_type(2)));
+          const s16x2 lo2 = {(short)lo, (short)lo}, hi2 = {(short)hi, (short)hi};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            uint32_t m = 0;
-            if (2 * d >= lo && 2 * d < hi) m |= 0xffffu;
-            if (2 * d + 1 >= lo && 2 * d + 1 < hi) m |= 0xffff0000u;
-            v[d] &= (int)m;
+            const s16x2 e = {(short)(2 * d), (short)(2 * d + 1)};
+            const s16x2 below_lo = (e - lo2) >> 15, below_hi = (e - hi2) >> 15;
+            v[d] &= __builtin_bit_cast(int, below_hi & ~below_lo);
           }
         }
       }

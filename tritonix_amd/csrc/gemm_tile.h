@@ -12,8 +12,8 @@
 //     wants k-contiguous lanes) with the transposing ds_read_b64_tr_b16/_b8;
 //   * XOR-swizzled 16-byte chunks so neither the DMA writes nor the fragment
 //     reads collide on LDS banks;
-//   * v_mfma_f32_32x32x16 (bf16/f16), v_mfma_i32_32x32x32_i8, or the 16x16
-//     shapes when a wave's tile is narrower than 32;
+//   * v_mfma_f32_16x16x32 (bf16/f16) and v_mfma_i32_16x16x64_i8 (the 32x32 shapes
+//     stay selectable through TileCfg::MI);
 //   * a 1-D grid whose block index is remapped XCD-first, then by the
 //     group-M order of tl.swizzle2d (tritonix/ops/matmul.py:70).
 #pragma once

@@ -23,7 +23,7 @@ __all__ = ["conv2d_forward", "conv2d_forward_kernel", "torch_conv2d_forward", "o
 _DTYPES = {torch.float16: _C.F16, torch.bfloat16: _C.BF16, torch.float32: _C.F32}
 
 # (BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M): the reference's candidates
-# (tritonix/ops/conv2d/forward.py:172-180) and two larger tiles this engine also builds
+# (tritonix/ops/conv2d/forward.py:172-180) and three larger tiles this engine also builds
 _CANDIDATE_CONFIGS = [
     (128, 128, 32, 8),
     (128, 64, 32, 8),
@@ -33,6 +33,7 @@ _CANDIDATE_CONFIGS = [
     (64, 128, 64, 8),
     (128, 64, 64, 8),
     (64, 64, 64, 8),
+    (64, 256, 64, 8),
     (128, 256, 64, 8),
     (256, 128, 64, 8),
 ]
