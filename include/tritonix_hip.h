@@ -205,8 +205,22 @@ typedef struct tnx_conv2d_args {
   int32_t bias_dtype;  /* TNX_F16 / TNX_BF16 / TNX_F32                              */
   int32_t block_pixels, block_cout, block_k; /* workgroup tile; 0 0 0 = built-in choice */
   int32_t group_pixels; /* pixel tiles per L2 group (tl.swizzle2d size_g); 0 = 8    */
+  int32_t loader;      /* tnx_conv_loader; 0 = the library chooses                   */
   void* stream;        /* hipStream_t; NULL = the null stream                       */
 } tnx_conv2d_args;
+
+/* How the slabs reach LDS.  Two kernels exist: one stages both operands through registers (any stride, padding,
+ * dilation, any c_in * filter_h * filter_w; tiles up to 256 x 128), the other is the GEMM kernel with a
+ * direct-to-LDS im2col loader (needs stride_w == 1, c_in * filter_h * filter_w a multiple of block_k = 64, a 16-byte
+ * aligned weight; tiles of 128 or 256 channels x 128 or 256 pixels).  With TNX_CONV_LOADER_AUTO and no tile given
+ * the library takes the direct-to-LDS kernel whenever the problem allows it and has enough tiles to fill the chip;
+ * with a tile given it takes it when the tile exists only there, or exists in both and the problem allows it.
+ * Asking for a loader the problem or tile does not allow returns TNX_E_UNSUPPORTED. */
+enum tnx_conv_loader {
+  TNX_CONV_LOADER_AUTO = 0,
+  TNX_CONV_LOADER_REGISTERS = 1,
+  TNX_CONV_LOADER_DMA = 2
+};
 
 /* Launch one conv2d forward.  Returns a tnx_status.  Asynchronous, allocates nothing. */
 int tnx_conv2d_forward(const tnx_conv2d_args* args);
@@ -222,7 +236,8 @@ void tnx_conv2d_output_size(const tnx_conv2d_args* args, int32_t* h_out, int32_t
 /* Fill block_pixels / block_cout / block_k / group_pixels with the built-in choice for this problem. */
 int tnx_conv2d_default_config(tnx_conv2d_args* args);
 
-/* Compiled conv2d tiles: count, and "dtype block_cout block_pixels block_k" of the i-th (static storage). */
+/* Compiled conv2d tiles: count, and "dtype block_cout block_pixels block_k loader" of the i-th (static storage;
+ * loader is "registers" or "dma"). */
 int tnx_conv2d_kernel_count(void);
 const char* tnx_conv2d_kernel_name(int i);
 

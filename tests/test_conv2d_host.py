@@ -56,20 +56,46 @@ def test_default_config_names_a_built_tile():
     lib = _C.load()
     built = set(_C.conv2d_kernel_names())
     assert len(built) >= 16
-    for kw in (dict(), dict(c_out=512, c_in=512), dict(c_out=8, c_in=3, filter_h=1, filter_w=1, pad_h=0, pad_w=0),
-               dict(batch=1, h_in=4, w_in=4)):
+    loaders = {_C.CONV_LOADER_REGISTERS: "registers", _C.CONV_LOADER_DMA: "dma"}
+    seen = set()
+    for kw in (dict(), dict(c_out=512, c_in=512, batch=32), dict(c_out=8, c_in=3, filter_h=1, filter_w=1, pad_h=0, pad_w=0),
+               dict(batch=1, h_in=4, w_in=4), dict(c_in=64, c_out=256, h_in=56, w_in=56, batch=32),
+               dict(c_in=64, c_out=128, h_in=28, w_in=28, batch=8), dict(c_in=64, c_out=128, stride_w=2)):
         a = _args(**kw)
         assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK
-        assert f"bf16 {a.block_cout} {a.block_pixels} {a.block_k}" in built
+        assert f"bf16 {a.block_cout} {a.block_pixels} {a.block_k} {loaders[a.loader]}" in built
         assert a.group_pixels == 8
         assert lib.tnx_conv2d_supported(ctypes.byref(a)) == _C.OK
+        seen.add((a.block_cout, a.block_pixels, loaders[a.loader]))
+    # c_in * 9 a multiple of 64 and unit stride along w: the direct-to-LDS kernel; 256 channels wide when that leaves
+    # two tiles per CU
+    assert (256, 128, "dma") in seen and (128, 128, "dma") in seen and (128, 64, "registers") in seen
+
+
+def test_loader_requests():
+    lib = _C.load()
+    ok = dict(c_in=64, c_out=128, block_pixels=128, block_cout=128, block_k=64)
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_DMA, **ok))) == _C.OK
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_REGISTERS, **ok))) == _C.OK
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=3, **ok))) == _C.E_INVALID
+    # stride along w, or c_in * R * S not a multiple of 64: only the register-staged kernel
+    for bad in (dict(stride_w=2), dict(c_in=16)):
+        kw = dict(ok, **bad)
+        assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_DMA, **kw))) == _C.E_UNSUPPORTED
+        assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_AUTO, **kw))) == _C.OK
+    # a tile only one of the two kernels has
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_DMA, c_in=64, block_pixels=64, block_cout=64,
+                                                       block_k=64))) == _C.E_UNSUPPORTED
 
 
 def test_every_reference_candidate_is_built():
     built = set(_C.conv2d_kernel_names())
     for bm, bn, bk, _ in conv._CANDIDATE_CONFIGS:
         for dt in ("bf16", "f16"):
-            assert f"{dt} {bn} {bm} {bk}" in built
+            assert f"{dt} {bn} {bm} {bk} registers" in built
+    for dt in ("bf16", "f16"):
+        for bc, bp in ((128, 128), (256, 128), (128, 256)):
+            assert f"{dt} {bc} {bp} 64 dma" in built
 
 
 def test_candidate_filter_follows_the_reference():

@@ -60,6 +60,55 @@ def test_conv2d_matches_the_oracle(name, dtype, device):
         assert ok, (name, dtype, cfg, err, rel)
 
 
+# geometries the direct-to-LDS kernel accepts: stride_w == 1, c_in * R * S a multiple of 64
+DMA_CASES = {
+    "1x1": (2, 64, 16, 16, 128, 1, 1, (1, 1), (0, 0), (1, 1), False),
+    "3x3_same": (2, 64, 16, 16, 128, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    "w_out_14_ragged_channels": (3, 64, 14, 14, 200, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    "w_out_7": (3, 128, 7, 7, 130, 3, 3, (1, 1), (1, 1), (1, 1), False),
+    "stride_h_2_dilated": (2, 64, 17, 13, 96, 3, 3, (2, 1), (2, 2), (2, 2), True),
+    "1x5_wide_pad": (2, 64, 9, 20, 64, 1, 5, (1, 1), (0, 3), (1, 1), True),
+    "no_pad": (1, 192, 10, 10, 256, 3, 3, (1, 1), (0, 0), (1, 1), True),
+    "5x5": (2, 64, 12, 12, 128, 5, 5, (1, 1), (2, 2), (1, 1), False),
+    "w_out_3": (2, 64, 3, 3, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),
+}
+DMA_TILES = [(128, 128, 64), (128, 256, 64), (256, 128, 64)]     # BLOCK_SIZE_M (pixels), BLOCK_SIZE_N (channels), BLOCK_SIZE_K
+
+
+@pytest.mark.parametrize("name", sorted(DMA_CASES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_direct_to_lds_loader_matches_the_oracle_and_the_register_kernel(name, dtype, device):
+    """Padding rows come from the buffer bound, padding columns from the in-LDS fix-up, the first and last chunk of the
+    tensor from the element-wise fill; every case has all three.  Both kernels add the same products in the same
+    order (block_k = 64, the same MFMA shape), so they must agree bit for bit."""
+    x, wt, b, stride, padding, dilation = _inputs(DMA_CASES[name], dtype, seed=len(name))
+    ref = _oracle(x, wt, b, stride, padding, dilation)
+    xd, wd, bd = x.to(device), wt.to(device), None if b is None else b.to(device)
+    regs = conv2d_forward(xd, wd, bd, stride, padding, dilation,
+                          config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, LOADER="registers"))
+    for bm, bn, bk in DMA_TILES:
+        cfg = dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, LOADER="dma")
+        out = conv2d_forward(xd, wd, bd, stride, padding, dilation, config=cfg)
+        ok, err, rel = oracle.within_tolerance(out, ref)
+        assert ok, (name, dtype, cfg, err, rel)
+        assert torch.equal(out, regs), (name, dtype, cfg)
+
+
+def test_loader_that_does_not_fit_is_refused(device):
+    x, wt, b, stride, padding, dilation = _inputs(CASES["1x1_stride2"], torch.bfloat16)
+    with pytest.raises(ValueError):           # stride_w == 2
+        conv2d_forward(x.to(device), wt.to(device), None, stride, padding, dilation,
+                       config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, LOADER="dma"))
+    x, wt, b, stride, padding, dilation = _inputs(CASES["3x3_same"], torch.bfloat16)
+    with pytest.raises(ValueError):           # c_in * 9 = 144 is not a multiple of 64
+        conv2d_forward(x.to(device), wt.to(device), None, stride, padding, dilation,
+                       config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, LOADER="dma"))
+    # the same tile without the demand falls back to the register-staged kernel
+    out = conv2d_forward(x.to(device), wt.to(device), None, stride, padding, dilation,
+                         config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64))
+    assert oracle.within_tolerance(out, _oracle(x, wt, None, stride, padding, dilation))[0]
+
+
 def test_float32_bias_and_no_bias_agree_with_the_oracle(device):
     x, wt, _, stride, padding, dilation = _inputs(CASES["3x3_same"], torch.bfloat16, seed=3)
     b32 = torch.randn(wt.shape[0], generator=torch.Generator().manual_seed(4))
@@ -148,6 +197,11 @@ def test_resnet_layer_at_size_against_the_vendor_routine_and_linearity(device):
     b = torch.randn(256, generator=g).bfloat16()
     xd, wd, bd = x.to(device), wt.to(device), b.to(device)
     out = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1))
+    regs = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1), config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64,
+                                                                         LOADER="registers"))
+    dma = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1), config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=256, BLOCK_SIZE_K=64,
+                                                                        LOADER="dma"))
+    assert torch.equal(regs, dma)
     for img in (0, 17, 31):
         ref = oracle.reference_conv2d(x[img:img + 1], wt, b, (1, 1), (1, 1), (1, 1))
         assert oracle.within_tolerance(out[img:img + 1], ref)[0]

@@ -25,6 +25,8 @@ SCHED_DEFAULT, SCHED_PERSISTENT, SCHED_SUPERBLOCK, SCHED_ATOMIC_REDUCE = 0, 1, 2
 # enum tnx_status
 OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP, E_STATIC_LIMIT = 0, 1, 2, 3, 4, 5, 6
 STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
+# enum tnx_conv_loader
+CONV_LOADER_AUTO, CONV_LOADER_REGISTERS, CONV_LOADER_DMA = 0, 1, 2
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
            "tnx_gemm_default_config", "tnx_tile_coords", "tnx_probe_mfma", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
@@ -60,7 +62,7 @@ class Conv2dArgs(ctypes.Structure):
         ("dil_h", ctypes.c_int32), ("dil_w", ctypes.c_int32),
         ("dtype", ctypes.c_int32), ("bias_dtype", ctypes.c_int32),
         ("block_pixels", ctypes.c_int32), ("block_cout", ctypes.c_int32), ("block_k", ctypes.c_int32),
-        ("group_pixels", ctypes.c_int32),
+        ("group_pixels", ctypes.c_int32), ("loader", ctypes.c_int32),
         ("stream", ctypes.c_void_p),
     ]
 

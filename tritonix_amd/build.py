@@ -27,6 +27,9 @@ ARCH = "gfx950"
 # packed-fp32 VALU ops are switched off on purpose for every device translation unit
 DEVICE_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                # the K loop is written as fully unrolled slots; with the conv2d loader in them the default limit on
+                # the size of a pragma-unrolled loop would leave one rolled (and the accumulators in scratch memory)
+                "-mllvm", "-pragma-unroll-threshold=100000",
                 "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 LDS_LIMIT = 160 * 1024

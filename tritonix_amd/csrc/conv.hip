@@ -2,6 +2,7 @@
 // Declarations and the reference interface they replace: include/tritonix_hip.h
 #include <hip/hip_runtime.h>
 #include <stdio.h>
+#include <string.h>
 
 #include "../../include/tritonix_hip.h"
 #include "conv_tile.h"
@@ -9,7 +10,20 @@
 
 using namespace tnx;
 
-extern "C" const ConvGroup* tnx_conv_groups(int* ngroups);  // generated
+extern "C" const ConvGroup* tnx_conv_groups(int* ngroups);      // generated
+extern "C" const KernelGroup* tnx_kernel_groups(int* ngroups);  // generated
+
+// the GEMM kernel's conv2d variant for this tile (four waves, three ring slots), or null
+static const KernelEntry* find_dma(int dtype, int bcout, int bpix, int bk) {
+  int ng = 0;
+  const KernelGroup* g = tnx_kernel_groups(&ng);
+  for (int i = 0; i < ng; ++i)
+    for (int j = 0; j < g[i].count; ++j) {
+      const KernelEntry& e = g[i].entries[j];
+      if (e.dtype == dtype && e.bm == bcout && e.bn == bpix && e.bk == bk && e.nw == 4 && e.stages == 3 && e.conv) return &e;
+    }
+  return nullptr;
+}
 
 static const ConvEntry* find_conv(int dtype, int bcout, int bpix, int bk) {
   int ng = 0;
@@ -46,6 +60,41 @@ static void builtin_tile(const tnx_conv2d_args* a, int64_t pixels, int* bcout, i
   *bk = gemm_k > 32 ? 64 : 32;
 }
 
+// Direct-to-LDS kernel: 256 channels x 128 pixels when that still leaves every CU two tiles, else 128 x 128.
+// Measured on 3x3 layers (batch 32): 256x128 538 against 389 TFLOP/s for 128x128 at 56x56 / 256 channels, 128x128
+// ahead of it at 28x28 / 128 channels (244 : 181) and 14x14 / 512 channels (352 : 282), and both well ahead of
+// the register-staged kernel (392, 162, 165) down to a few dozen tiles.
+static bool builtin_dma_tile(const tnx_conv2d_args* a, int h_out, int w_out, int* bcout, int* bpix, int* bk) {
+  const int64_t cols = (int64_t)a->batch * h_out * ((w_out + 7) / 8 * 8);
+  const int64_t t256 = ((cols + 127) / 128) * (((int64_t)a->c_out + 255) / 256);
+  const int64_t t128 = ((cols + 127) / 128) * (((int64_t)a->c_out + 127) / 128);
+  *bpix = 128;
+  *bk = 64;
+  if (a->c_out > 128 && t256 >= 512 && find_dma(a->dtype, 256, 128, 64)) {
+    *bcout = 256;
+    return true;
+  }
+  if (a->c_out > 64 && t128 >= 32 && find_dma(a->dtype, 128, 128, 64)) {
+    *bcout = 128;
+    return true;
+  }
+  return false;
+}
+
+// `rows` taps further along k = (c_in, fh, fw): rows = sc * (R*S) + sh * S + sw
+static void tap_step(const tnx_conv2d_args* a, int rows, int hw_in, int* step_dw, int* step_dh, int* step_koff, int* lim_w,
+                     int* lim_h, int* adj_w, int* adj_h) {
+  const int rs = a->filter_h * a->filter_w;
+  const int sc = rows / rs, sh = (rows % rs) / a->filter_w, sw = rows % a->filter_w;
+  *step_dw = sw * a->dil_w;
+  *step_dh = sh * a->dil_h;
+  *step_koff = sc * hw_in + *step_dh * a->w_in + *step_dw;
+  *lim_w = a->filter_w * a->dil_w;
+  *lim_h = a->filter_h * a->dil_h;
+  *adj_w = a->dil_h * a->w_in - *lim_w;          // dw wraps: one filter row down
+  *adj_h = hw_in - *lim_h * a->w_in;             // dh wraps: next input channel
+}
+
 // everything about the problem except the tile
 static int check_problem(const tnx_conv2d_args* a, int32_t* h_out, int32_t* w_out) {
   if (!a) return TNX_E_INVALID;
@@ -69,22 +118,63 @@ static int check_problem(const tnx_conv2d_args* a, int32_t* h_out, int32_t* w_ou
   return TNX_OK;
 }
 
-static int resolve(const tnx_conv2d_args* a, const ConvEntry** entry, ConvParams* p, unsigned* grid) {
+// what the direct-to-LDS kernel needs of the problem (not of the tile)
+static bool dma_problem_ok(const tnx_conv2d_args* a, int h_out, int w_out, bool inspect_ptrs) {
+  const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
+  const int64_t wp = (w_out + 7) / 8 * 8;
+  if (a->stride_w != 1 || gemm_k % 64 != 0) return false;
+  if ((int64_t)a->batch * h_out * wp >= (1ll << 31) - 4096) return false;
+  if (inspect_ptrs && ((uintptr_t)a->weight & 15)) return false;
+  // per-lane DMA offsets of the weight slab are 32-bit
+  if (256 * gemm_k * 2 >= (1ll << 32)) return false;
+  return true;
+}
+
+struct Resolved {
+  const ConvEntry* reg;      // register-staged kernel, or
+  const KernelEntry* dma;    // the GEMM kernel's conv2d variant
+  int bcout, bpix, bk;
+  int h_out, w_out;
+};
+
+static int resolve(const tnx_conv2d_args* a, Resolved* r, bool inspect_ptrs) {
   int32_t h_out = 0, w_out = 0;
   const int st = check_problem(a, &h_out, &w_out);
   if (st != TNX_OK) return st;
+  if (a->loader < TNX_CONV_LOADER_AUTO || a->loader > TNX_CONV_LOADER_DMA) return TNX_E_INVALID;
   const int64_t pixels = (int64_t)a->batch * h_out * w_out;
+  const bool dma_ok = dma_problem_ok(a, h_out, w_out, inspect_ptrs);
   int bcout = a->block_cout, bpix = a->block_pixels, bk = a->block_k;
-  if (bcout == 0 && bpix == 0 && bk == 0) builtin_tile(a, pixels, &bcout, &bpix, &bk);
+  const bool builtin = bcout == 0 && bpix == 0 && bk == 0;
+  bool want_dma = a->loader == TNX_CONV_LOADER_DMA;
+  if (builtin) {
+    if (a->loader != TNX_CONV_LOADER_REGISTERS && dma_ok && builtin_dma_tile(a, h_out, w_out, &bcout, &bpix, &bk)) want_dma = true;
+    else if (want_dma) return TNX_E_UNSUPPORTED;
+    else builtin_tile(a, pixels, &bcout, &bpix, &bk);
+  }
   if (bcout <= 0 || bpix <= 0 || bk <= 0) return TNX_E_INVALID;
-  if (2ll * ((int64_t)bcout * bk + (int64_t)bk * bpix) * 2 > TNX_LDS_LIMIT_BYTES) return TNX_E_LDS;
-  const ConvEntry* e = find_conv(a->dtype, bcout, bpix, bk);
-  if (!e) return TNX_E_UNSUPPORTED;
-  const int64_t tiles_pix = (pixels + bpix - 1) / bpix, tiles_cout = ((int64_t)a->c_out + bcout - 1) / bcout;
-  if (tiles_pix * tiles_cout >= (1ll << 31)) return TNX_E_UNSUPPORTED;
-  *entry = e;
-  if (!p) return TNX_OK;
+  if (2ll * ((int64_t)bcout * bk + (int64_t)bk * bpix) * 2 > TNX_LDS_LIMIT_BYTES) return TNX_E_LDS;   // two slots: the smaller of the two kernels
+  const ConvEntry* reg = find_conv(a->dtype, bcout, bpix, bk);
+  const KernelEntry* dma = find_dma(a->dtype, bcout, bpix, bk);
+  if (!builtin && a->loader == TNX_CONV_LOADER_AUTO) want_dma = dma && dma_ok;
+  if (want_dma && !(dma && dma_ok)) {
+    if (a->loader == TNX_CONV_LOADER_DMA) return TNX_E_UNSUPPORTED;
+    want_dma = false;
+  }
+  if (!want_dma && !reg) return TNX_E_UNSUPPORTED;
+  const int64_t cols = want_dma ? (int64_t)a->batch * h_out * ((w_out + 7) / 8 * 8) : pixels;
+  if (((cols + bpix - 1) / bpix) * (((int64_t)a->c_out + bcout - 1) / bcout) >= (1ll << 31)) return TNX_E_UNSUPPORTED;
+  r->reg = want_dma ? nullptr : reg;
+  r->dma = want_dma ? dma : nullptr;
+  r->bcout = bcout; r->bpix = bpix; r->bk = bk;
+  r->h_out = h_out; r->w_out = w_out;
+  return TNX_OK;
+}
 
+static void fill_registers(const tnx_conv2d_args* a, const Resolved& r, ConvParams* p, unsigned* grid) {
+  const int h_out = r.h_out, w_out = r.w_out, bk = r.bk;
+  const int64_t pixels = (int64_t)a->batch * h_out * w_out;
+  const int64_t tiles_pix = (pixels + r.bpix - 1) / r.bpix, tiles_cout = ((int64_t)a->c_out + r.bcout - 1) / r.bcout;
   const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
   const int64_t x_elems = (int64_t)a->batch * a->c_in * a->h_in * a->w_in;
   p->x = (const uint8_t*)a->input;
@@ -106,18 +196,7 @@ static int resolve(const tnx_conv2d_args* a, const ConvEntry** entry, ConvParams
   p->div_w_out = make_fastdiv((uint32_t)w_out);
   p->div_rs = make_fastdiv((uint32_t)(a->filter_h * a->filter_w));
   p->div_s = make_fastdiv((uint32_t)a->filter_w);
-  {
-    // block_k = sc * (R*S) + sh * S + sw
-    const int rs = a->filter_h * a->filter_w;
-    const int sc = bk / rs, sh = (bk % rs) / a->filter_w, sw = bk % a->filter_w;
-    p->step_dw = sw * a->dil_w;
-    p->step_dh = sh * a->dil_h;
-    p->step_koff = sc * p->hw_in + p->step_dh * a->w_in + p->step_dw;
-    p->lim_w = a->filter_w * a->dil_w;
-    p->lim_h = a->filter_h * a->dil_h;
-    p->adj_w = a->dil_h * a->w_in - p->lim_w;          // dw wraps: one filter row down
-    p->adj_h = p->hw_in - p->lim_h * a->w_in;          // dh wraps: next input channel
-  }
+  tap_step(a, bk, p->hw_in, &p->step_dw, &p->step_dh, &p->step_koff, &p->lim_w, &p->lim_h, &p->adj_w, &p->adj_h);
   p->tiles_cout = (int)tiles_cout;
   p->tiles_pix = (int)tiles_pix;
   p->group = a->group_pixels > 0 ? a->group_pixels : 8;
@@ -126,38 +205,87 @@ static int resolve(const tnx_conv2d_args* a, const ConvEntry** entry, ConvParams
   p->y_vec_ok = p->hw_out % 4 == 0 && ((uintptr_t)a->output & 7) == 0;
   p->flat = a->filter_h == 1 && a->filter_w == 1 && a->stride_h == 1 && a->stride_w == 1 && a->pad_h == 0 && a->pad_w == 0;
   *grid = (unsigned)(tiles_pix * tiles_cout);
-  return TNX_OK;
+}
+
+// GemmParams of the GEMM kernel's conv2d variant: m = c_out, n = padded pixel index, k = c_in * R * S
+static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p, unsigned* grid) {
+  const int h_out = r.h_out, w_out = r.w_out;
+  const int wp = (w_out + 7) / 8 * 8;
+  const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
+  const int64_t n_total = (int64_t)a->batch * h_out * wp;
+  memset(p, 0, sizeof *p);
+  p->a = (const uint8_t*)a->weight;
+  p->b = (const uint8_t*)a->input;
+  p->c = (uint8_t*)a->output;
+  p->m = a->c_out; p->n = n_total; p->k = gemm_k;
+  p->sam = gemm_k; p->sak = 1;
+  p->tiles_m = (int)(((int64_t)a->c_out + r.bcout - 1) / r.bcout);
+  p->tiles_n = (int)((n_total + r.bpix - 1) / r.bpix);
+  p->group_m = 8;            // with one or two channel tiles: the channel tiles of one pixel tile run side by side
+  p->split_k = 1;
+  p->ktiles_per_split = (int)(gemm_k / r.bk);
+  p->out_dtype = a->dtype;
+  ConvGeom& g = p->cv;
+  g.h_in = a->h_in; g.w_in = a->w_in; g.c_out = a->c_out; g.h_out = h_out; g.w_out = w_out; g.wp = wp;
+  g.stride_h = a->stride_h; g.pad_h = a->pad_h; g.pad_w = a->pad_w;
+  g.hw_in = a->h_in * a->w_in;
+  g.chw_in = a->c_in * g.hw_in;
+  g.n_total = (int)n_total;
+  g.x_bytes = (uint32_t)((int64_t)a->batch * g.chw_in * 2);
+  g.div_hwp = make_fastdiv((uint32_t)(h_out * wp));
+  g.div_wp = make_fastdiv((uint32_t)wp);
+  g.rs = a->filter_h * a->filter_w;
+  g.fw = a->filter_w;
+  g.div_rs = make_fastdiv((uint32_t)g.rs);
+  g.div_s = make_fastdiv((uint32_t)g.fw);
+  g.dil_h = a->dil_h; g.dil_w = a->dil_w;
+  // k rows one DMA op of the workgroup covers: 256 lanes x 16 bytes over rows of block_pixels * 2 bytes
+  const int rows_per_op = 4 * 64 / (r.bpix * 2 / 16);
+  tap_step(a, rows_per_op, g.hw_in, &g.step_dw, &g.step_dh, &g.step_koff, &g.lim_w, &g.lim_h, &g.adj_w, &g.adj_h);
+  g.bias = (const uint8_t*)a->bias;
+  g.bias_dtype = a->bias_dtype;
+  *grid = (unsigned)((int64_t)p->tiles_m * p->tiles_n);
 }
 
 extern "C" int tnx_conv2d_supported(const tnx_conv2d_args* a) {
-  const ConvEntry* e = nullptr;
-  return resolve(a, &e, nullptr, nullptr);
+  Resolved r;
+  return resolve(a, &r, false);
 }
 
 extern "C" int tnx_conv2d_default_config(tnx_conv2d_args* a) {
-  int32_t h_out = 0, w_out = 0;
-  const int st = check_problem(a, &h_out, &w_out);
+  if (!a) return TNX_E_INVALID;
+  tnx_conv2d_args tmp = *a;
+  tmp.block_cout = tmp.block_pixels = tmp.block_k = 0;
+  Resolved r;
+  const int st = resolve(&tmp, &r, false);
   if (st != TNX_OK) return st;
-  int bcout, bpix, bk;
-  builtin_tile(a, (int64_t)a->batch * h_out * w_out, &bcout, &bpix, &bk);
-  a->block_cout = bcout;
-  a->block_pixels = bpix;
-  a->block_k = bk;
+  a->block_cout = r.bcout;
+  a->block_pixels = r.bpix;
+  a->block_k = r.bk;
   a->group_pixels = 8;
+  a->loader = r.dma ? TNX_CONV_LOADER_DMA : TNX_CONV_LOADER_REGISTERS;
   return TNX_OK;
 }
 
 extern "C" int tnx_conv2d_forward(const tnx_conv2d_args* a) {
-  const ConvEntry* e = nullptr;
-  ConvParams p;
-  unsigned grid = 0;
-  const int st = resolve(a, &e, &p, &grid);
+  Resolved r;
+  const int st = resolve(a, &r, true);
   if (st != TNX_OK) return st;
   if (!a->input || !a->weight || !a->output) return TNX_E_INVALID;
   // 16-bit elements are read and written as such
   if (((uintptr_t)a->input & 1) || ((uintptr_t)a->weight & 1) || ((uintptr_t)a->output & 1)) return TNX_E_INVALID;
   if (a->bias && ((uintptr_t)a->bias & (a->bias_dtype == TNX_F32 ? 3 : 1))) return TNX_E_INVALID;
-  const hipError_t err = e->launch(p, grid, (hipStream_t)a->stream);
+  unsigned grid = 0;
+  hipError_t err;
+  if (r.dma) {
+    GemmParams p;
+    fill_dma(a, r, &p, &grid);
+    err = r.dma->conv(p, grid, (hipStream_t)a->stream);
+  } else {
+    ConvParams p;
+    fill_registers(a, r, &p, &grid);
+    err = r.reg->launch(p, grid, (hipStream_t)a->stream);
+  }
   if (err != hipSuccess) {
     note_hip_error((int)err);
     return TNX_E_HIP;
@@ -165,23 +293,30 @@ extern "C" int tnx_conv2d_forward(const tnx_conv2d_args* a) {
   return TNX_OK;
 }
 
-extern "C" int tnx_conv2d_kernel_count(void) {
-  int ng = 0, n = 0;
+// register-staged tiles first, then the GEMM kernel's conv2d variants
+template <class F> static void each_conv_kernel(F f) {
+  int ng = 0;
   const ConvGroup* g = tnx_conv_groups(&ng);
-  for (int i = 0; i < ng; ++i) n += g[i].count;
+  for (int i = 0; i < ng; ++i)
+    for (int j = 0; j < g[i].count; ++j) f(g[i].entries[j].dtype, g[i].entries[j].block_cout, g[i].entries[j].block_pix, g[i].entries[j].block_k, false);
+  const KernelGroup* k = tnx_kernel_groups(&ng);
+  for (int i = 0; i < ng; ++i)
+    for (int j = 0; j < k[i].count; ++j)
+      if (k[i].entries[j].conv) f(k[i].entries[j].dtype, k[i].entries[j].bm, k[i].entries[j].bn, k[i].entries[j].bk, true);
+}
+
+extern "C" int tnx_conv2d_kernel_count(void) {
+  int n = 0;
+  each_conv_kernel([&](int, int, int, int, bool) { ++n; });
   return n;
 }
 
 extern "C" const char* tnx_conv2d_kernel_name(int idx) {
   static thread_local char buf[64];
-  int ng = 0, n = 0;
-  const ConvGroup* g = tnx_conv_groups(&ng);
-  for (int i = 0; i < ng; ++i)
-    for (int j = 0; j < g[i].count; ++j, ++n)
-      if (n == idx) {
-        const ConvEntry& e = g[i].entries[j];
-        snprintf(buf, sizeof buf, "%s %d %d %d", e.dtype == TNX_F16 ? "f16" : "bf16", e.block_cout, e.block_pix, e.block_k);
-        return buf;
-      }
-  return "";
+  int n = 0;
+  buf[0] = 0;
+  each_conv_kernel([&](int dtype, int bc, int bp, int bk, bool dma) {
+    if (n++ == idx) snprintf(buf, sizeof buf, "%s %d %d %d %s", dtype == TNX_F16 ? "f16" : "bf16", bc, bp, bk, dma ? "dma" : "registers");
+  });
+  return buf;
 }

@@ -17,27 +17,6 @@
 
 namespace tnx {
 
-// n / d for 0 <= n < 2^31 by multiply-high and shift (d >= 1); built on the host.
-struct FastDiv {
-  uint32_t mul, shift;
-};
-inline FastDiv make_fastdiv(uint32_t d) {
-  FastDiv f = {0u, 0u};
-  if (d <= 1) return f;
-  uint32_t s = 0;
-  while ((1ull << s) < d) ++s;
-  f.shift = s;
-  f.mul = (uint32_t)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
-  return f;
-}
-__host__ __device__ __forceinline__ uint32_t fd_div(uint32_t n, FastDiv f) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  return (__umulhi(n, f.mul) + n) >> f.shift;
-#else
-  return (uint32_t)((((uint64_t)n * f.mul) >> 32) + n) >> f.shift;
-#endif
-}
-
 struct ConvParams {
   const uint8_t* x;       // [batch, c_in, h_in, w_in]
   const uint8_t* w;       // [c_out, c_in, fh, fw]  ==  [c_out, gemm_k] row-major
@@ -71,17 +50,6 @@ struct ConvEntry {
 struct ConvGroup {
   ConvEntry* entries;
   int count;
-};
-
-__device__ __forceinline__ float bias_value(const uint8_t* bias, int row, int dtype) {
-  if (dtype == DT_F32) return ((const float*)bias)[row];
-  if (dtype == DT_F16) return (float)((const _Float16*)bias)[row];
-  return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)bias)[row] << 16);
-}
-
-// 16 bytes from an address that is only 2-byte aligned
-struct __attribute__((packed, aligned(2))) Loose16 {
-  i32x4 v;
 };
 
 // C = TileCfg<T, block_cout, block_pix, block_k, 4 waves, 2 slots>

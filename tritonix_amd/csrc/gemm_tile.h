@@ -36,6 +36,47 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 enum { DT_F16 = 0, DT_BF16 = 1, DT_I8 = 2, DT_I32 = 3, DT_F32 = 4 };
 enum { EPI_NONE = 0, EPI_GLU_SILU = 1, EPI_GLU_SIGMOID = 2, EPI_GLU_IDENTITY = 3 };
 
+// n / d for 0 <= n < 2^31 by multiply-high and shift (d >= 1); built on the host.
+struct FastDiv {
+  uint32_t mul, shift;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f = {0u, 0u};
+  if (d <= 1) return f;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  f.shift = s;
+  f.mul = (uint32_t)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
+  return f;
+}
+__host__ __device__ __forceinline__ uint32_t fd_div(uint32_t n, FastDiv f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (__umulhi(n, f.mul) + n) >> f.shift;
+#else
+  return (uint32_t)((((uint64_t)n * f.mul) >> 32) + n) >> f.shift;
+#endif
+}
+
+// Geometry of a conv2d forward run on the GEMM kernel (gemm_tile_kernel<..., CONV>): A is the KCRS weight as
+// [c_out, c_in*R*S], the B operand is generated from the NCHW input by the DMA loader, column n of the product is
+// pixel (image, h_out, w) of a pixel index space whose rows are `wp` wide (w_out rounded up to 8, so that a 16-byte
+// chunk of 8 pixels never leaves its output row; the pixels w >= w_out of a row are computed and dropped).
+struct ConvGeom {
+  int h_in, w_in, c_out, h_out, w_out, wp;
+  int stride_h, pad_h, pad_w;
+  int hw_in, chw_in;               // h_in*w_in, c_in*h_in*w_in
+  int n_total;                     // batch * h_out * wp
+  uint32_t x_bytes;                // size of the input tensor
+  FastDiv div_hwp, div_wp;         // by h_out*wp, by wp
+  FastDiv div_rs, div_s;           // by R*S, by S
+  int rs, fw, dil_h, dil_w;
+  // one DMA op further along k (the rows one op of the workgroup covers): what is added to a tap's (dw, dh, element
+  // offset), the limits at which dw and dh wrap, and what a wrap adds to the element offset
+  int step_dw, step_dh, step_koff, lim_w, lim_h, adj_w, adj_h;
+  const uint8_t* bias;             // [c_out] or null
+  int bias_dtype;
+};
+
 struct GemmParams {
   const uint8_t* a;
   const uint8_t* b;
@@ -56,6 +97,7 @@ struct GemmParams {
   bool b_once;            // every element of B is read by exactly one workgroup (one tile row): stream it non-temporally
   int tile_order;         // 0: XCD remap + tl.swizzle2d(group_m); 1: 16x16 super-blocks in serpentine order (superblock_order)
   int atomic_reduce;      // split-K: slices are added into one fp32/int32 copy with device-scope atomics instead of being kept apart
+  ConvGeom cv;            // only read by the CONV kernels
 };
 
 // ---------------------------------------------------------------------------
@@ -697,6 +739,94 @@ __device__ __forceinline__ bool splitk_arrive(ACC (&acc)[C::TM][C::TN], uint8_t*
   return last;
 }
 
+__device__ __forceinline__ float bias_value(const uint8_t* bias, int row, int dtype) {
+  if (dtype == DT_F32) return ((const float*)bias)[row];
+  if (dtype == DT_F16) return (float)((const _Float16*)bias)[row];
+  return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)bias)[row] << 16);
+}
+
+// 16 bytes from an address that is only 2-byte aligned
+struct __attribute__((packed, aligned(2))) Loose16 {
+  i32x4 v;
+};
+
+
+// Epilogue of the CONV kernels: rows are output channels, columns are pixels of the padded pixel index space.  Same
+// pass through the wave's LDS strip as epilogue_store; a 16-byte chunk is 8 pixels of one output row, so it is one
+// run of the NCHW output (cut at w_out: the pixels past it exist only in the index space).  Bias is added in fp32.
+template <class T, class C, class O, class ACC>
+__device__ __forceinline__ void epilogue_store_conv(ACC (&acc)[C::TM][C::TN], uint8_t* ybase, uint32_t lds_strip, int lane,
+                                                    int gm0, int gn0, const ConvGeom& g) {
+  typedef Pack16<O, float, false> PK;
+  typedef typename PK::raw raw;
+  typedef float acc4 __attribute__((ext_vector_type(4)));
+  constexpr int MI = C::MI;
+  constexpr int NGRP = C::ACC_N / 4;
+  constexpr int PITCH = EpiStage<C>::PITCH;
+  constexpr int ROWS = EpiStage<C>::ROWS;
+  constexpr int CPRW = C::WTN / PK::OUTV;
+  constexpr int ITERS = (ROWS * CPRW + 63) / 64;
+  constexpr int UNR = ITERS % 4 == 0 ? 4 : (ITERS % 2 == 0 ? 2 : 1);
+  static_assert(EpiStage<C>::RB == 1 && PK::OUTV == 8, "one row-block per pass, 8 outputs per chunk");
+  raw* yp = (raw*)ybase;
+  const uint32_t wbase = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+    if (gm0 + i * MI >= g.c_out) break;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int q = 0; q < NGRP; ++q)
+        *TNX_LDS(acc4, wbase + (j * MI + q * 8) * 4) =
+            acc4{acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+#pragma unroll 1
+    for (int it0 = 0; it0 < ITERS; it0 += UNR) {
+      float f[UNR][8];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int q = (it0 + u) * 64 + lane;
+        int row = q / CPRW;
+        const int cc = q % CPRW;
+        if (ROWS * CPRW % 64 != 0 && row >= ROWS) row = ROWS - 1;
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+          const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * 8 + 4 * x) * 4);
+          __builtin_memcpy(&f[u][4 * x], &v, 16);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int q = (it0 + u) * 64 + lane;
+        const int row = q / CPRW, cc = q % CPRW;
+        const int gm = gm0 + i * MI + row;
+        const int gc = gn0 + cc * 8;
+        if ((ROWS * CPRW % 64 != 0 && row >= ROWS) || gm >= g.c_out || gc >= g.n_total) continue;
+        const int img = (int)fd_div((uint32_t)gc, g.div_hwp);
+        const int r = gc - img * (g.h_out * g.wp);
+        const int ho = (int)fd_div((uint32_t)r, g.div_wp);
+        const int wq = r - ho * g.wp;
+        const int valid = g.w_out - wq;              // pixels of this chunk that exist
+        if (valid <= 0) continue;
+        const float bv = g.bias ? bias_value(g.bias, gm, g.bias_dtype) : 0.0f;
+        raw out[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) out[x] = O::cvt(f[u][x] + bv);
+        raw* dst = yp + (((int64_t)img * g.c_out + gm) * g.h_out + ho) * g.w_out + wq;
+        if (valid >= 8) {
+          Loose16 v;
+          __builtin_memcpy(&v, out, 16);
+          *(Loose16*)dst = v;
+        } else {
+#pragma unroll 1
+          for (int x = 0; x < valid; ++x) dst[x] = out[x];
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+  }
+}
+
 template <bool B> struct BoolTag { static constexpr bool value = B; };
 template <int V> struct IntTag { static constexpr int value = V; };
 
@@ -706,13 +836,25 @@ template <int V> struct IntTag { static constexpr int value = V; };
 // BT: B is k-contiguous (element (k, n) at b + n * stride_bn + k, the layout of `x @ w.t()` with a
 // row-major weight): its slab sits in LDS as BN rows of BK elements exactly like the A slab, and its
 // fragments are read with plain ds_read_b128 -- no transposing read is needed.
-template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false>
+// CONV: conv2d forward (ConvGeom): A is the weight, the B slab is gathered from the NCHW input by the DMA loader --
+// one 16-byte raw-buffer load per chunk of 8 pixels from an address that is only 2-byte aligned, with an
+// out-of-range offset (the buffer bound answers zero) for chunks whose input row lies in the padding.  The elements
+// of a chunk that fall into the left / right padding have to be zeroed in LDS afterwards, by the wave that loaded
+// them.  Done between the wait for the loads and the barrier that publishes the slab, that fix-up sits on the
+// critical path of every K slab (measured: 340 instead of 630 TFLOP/s on a 3x3 layer), so the ring has three slots
+// and a slab spends one whole period between landing and being read: slab t+3 is issued during period t, has
+// landed when period t+1 starts (every wave waits for all of its own loads there, as with two slots), is fixed
+// during period t+1 -- one read-modify-write of the chunk per op, slotted behind that period's first MFMAs -- and
+// is published by barrier t+2, before whose period nothing reads it.  16-bit types, stride_w == 1, k % BK == 0.
+template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false, bool CONV = false>
 __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
   constexpr int MI = C::MI, TM = C::TM, TN = C::TN;
   static_assert(C::VALID, "tile configuration not supported by this kernel");
   static_assert(!PERSIST || FAST, "the persistent kernel is built with the DMA loader only");
   static_assert(!BT || (FAST && C::B_LOADS % NW == 0), "the k-contiguous B variant is built with the DMA loader only");
+  static_assert(!CONV || (FAST && !PERSIST && !BT && ES == 2 && STAGES == 3 && MI == 16 && (NW * 64) % C::CPR_B == 0),
+                "the conv2d variant: DMA loader, 16-bit types, three ring slots");
   typedef Mma<T, MI> MMA;
   typedef typename MMA::acc_t acc_t;
   typedef typename T::acc_s acc_s;
@@ -720,7 +862,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // one workgroup per tile: the epilogue strips are laid over the ring once the K loop is done.
   // persistent: the ring is refilled for the next tile during the epilogue, so the strips follow it.
   constexpr int RING_OR_STRIPS = C::LDS_BYTES > EpiStage<C>::BYTES ? C::LDS_BYTES : EpiStage<C>::BYTES;
-  constexpr int SMEM_BYTES = PERSIST ? C::LDS_BYTES + PairStrip<C>::BYTES : RING_OR_STRIPS;
+  // CONV: behind the ring, a table of the 81 16-byte masks that keep elements [lo, hi) of a chunk (0 <= lo, hi <= 8)
+  constexpr int CV_TABLE_BYTES = CONV ? 81 * 16 : 0;
+  constexpr int SMEM_BYTES = (PERSIST ? C::LDS_BYTES + PairStrip<C>::BYTES : RING_OR_STRIPS) + CV_TABLE_BYTES;
   static_assert(SMEM_BYTES <= 163840, "LDS budget of one CU exceeded");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[SMEM_BYTES];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
@@ -777,6 +921,36 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // current one has run, so the epilogue keeps its own copy of the origin.)
   int64_t m0 = 0, n0 = 0;
   uint32_t a_voff[C::A_LPW], b_voff[C::B_LPW];
+  // CONV: a lane's B ops all fetch the same 16-byte LDS column slot; the pixel chunk that lands there is one of
+  // two (the LDS swizzle moves it by two chunks depending on the k row): element offset of (image, channel 0,
+  // h0, w0) and the packed (h0, w0) for both, (h0, w0) being the input position of filter tap (0, 0).  Pixels past
+  // the end get h0 = -32768, which no tap brings back into the image.  One running filter tap per lane, advanced
+  // after every op by the k rows the workgroup covers per op (additions and wrap-arounds only).
+  constexpr int CONV_STEP = (NW * 64) / C::CPR_B;          // k rows covered by one B op of the workgroup
+  const int cv_r0 = tid / C::CPR_B;                          // k row of this lane in the first op of a slab
+  int pix_off0 = 0, pix_off1 = 0, pix_hw0 = 0, pix_hw1 = 0;   // (scalars, not arrays: an array indexed by a run-time bit is moved to LDS by the compiler)
+  int tap_dh = 0, tap_dw = 0;
+  uint32_t tap_off = 0;
+  uint32_t cv_fix[CONV ? C::B_LPW : 1];                      // per op of the slab in flight: what its fix-up has to do
+  bool cv_pending = false;
+  uint32_t cv_dst = 0;
+  constexpr uint32_t CV_OUTSIDE = 0xffffffffu, CV_NOFIX = 8u * 16u;   // a note is the byte offset of mask (lo, hi) in the table: (lo * 9 + hi) * 16
+  const uint32_t cv_table = lds0 + RING_OR_STRIPS;
+  i32x4 cv_rsrc = {0, 0, 0, 0};
+  if constexpr (CONV) {
+    if (tid < 81) {
+      const int lo = tid / 9, hi = tid % 9;
+      i32x4 m;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        m[d] = (int)((2 * d >= lo && 2 * d < hi ? 0xffffu : 0u) | (2 * d + 1 >= lo && 2 * d + 1 < hi ? 0xffff0000u : 0u));
+      *TNX_LDS(i32x4, cv_table + tid * 16) = m;
+    }
+    __syncthreads();
+    const uint64_t xa = (uint64_t)(uintptr_t)p.b;
+    cv_rsrc = i32x4{(int)__builtin_amdgcn_readfirstlane((uint32_t)xa), (int)(__builtin_amdgcn_readfirstlane((uint32_t)(xa >> 32)) & 0xffff),
+                    (int)__builtin_amdgcn_readfirstlane(p.cv.x_bytes), 0x00020000};
+  }
   const uint8_t* a_sbase = p.a;
   const uint8_t* b_sbase = p.b;
   auto place_tile = [&](int tile_m, int tile_n) __attribute__((always_inline)) {
@@ -796,9 +970,36 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         int64_t r = row < mrem ? row : mrem;
         a_voff[q] = (uint32_t)(r * lda * ES + c * 16);
       }
+      if constexpr (CONV) {
+        const ConvGeom& g = p.cv;
+        const int cs = tid % C::CPR_B;
+        const int c0 = cs ^ C::swzB(cv_r0 & 7);              // rows 0-7: the swizzle without its pass term
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const int n = (int)n0 + ((c0 ^ (v << 1)) << 3);
+          int off = 0, h0 = -32768, w0 = 0;
+          if (n < g.n_total) {
+            const int img = (int)fd_div((uint32_t)n, g.div_hwp);
+            const int r = n - img * (g.h_out * g.wp);
+            const int ho = (int)fd_div((uint32_t)r, g.div_wp);
+            h0 = ho * g.stride_h - g.pad_h;
+            w0 = (r - ho * g.wp) - g.pad_w;
+            off = img * g.chw_in + h0 * g.w_in + w0;
+          }
+          const int hw = (int)(((uint32_t)h0 << 16) | ((uint32_t)w0 & 0xffffu));
+          if (v == 0) { pix_off0 = off; pix_hw0 = hw; } else { pix_off1 = off; pix_hw1 = hw; }
+        }
+        // the tap of k row cv_r0 (the K loop starts at k = 0: these kernels are never cut along K)
+        const int cin = (int)fd_div((uint32_t)cv_r0, g.div_rs);
+        const int r = cv_r0 - cin * g.rs;
+        const int th = (int)fd_div((uint32_t)r, g.div_s);
+        tap_dh = th * g.dil_h;
+        tap_dw = (r - th * g.fw) * g.dil_w;
+        tap_off = (uint32_t)(cin * g.hw_in + tap_dh * g.w_in + tap_dw);
+      }
       const int64_t nrem = p.n - 1 - n0;  // last valid column inside this tile
 #pragma unroll
-      for (int q = 0; q < C::B_LPW; ++q) {
+      for (int q = 0; q < (CONV ? 0 : C::B_LPW); ++q) {
         int P = (q * NW + wave) * 64 + lane;
         if (BT) {
           // rows of the slab are columns of B: same chunk layout and swizzle as the A slab
@@ -851,9 +1052,135 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
   };
 
+  // CONV: byte offset of B op qb's chunk inside the input (or CV_OUTSIDE), its fix-up note, and the tap moved on
+  uint32_t cv_voff = 0;
+  auto conv_prepare = [&](int qb, uint32_t stage_base) __attribute__((always_inline)) {
+    const ConvGeom& g = p.cv;
+    const int row = qb * CONV_STEP + cv_r0;
+    const bool second = ((row >> 3) ^ (row >> 4)) & 1;      // the pass term of swzB
+    const int off = second ? pix_off1 : pix_off0, hw = second ? pix_hw1 : pix_hw0;
+    const int h0 = hw >> 16, w0 = (int)(int16_t)(hw & 0xffff);
+    const int o = off + (int)tap_off;
+    int lo = -(w0 + tap_dw), hi = g.w_in - (w0 + tap_dw);    // elements [lo, hi) of the chunk lie inside the input row
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > 8 ? 8 : hi;
+    const bool ok = (uint32_t)(h0 + tap_dh) < (uint32_t)g.h_in && lo < hi;
+    // A chunk that starts before the tensor (first row of the first image, left padding) or ends after it (last
+    // row of the last image, right padding) cannot be fetched whole -- the buffer bound drops every dword that is
+    // not entirely inside, valid elements included: it is loaded as zeros and its inside elements are written by
+    // the fix-up.  -o resp. (elements - o) is below 8 in those cases and is all the fix-up needs to find them.
+    const int x_elems = (int)(g.x_bytes >> 1);
+    const bool before = o < 0, after = o > x_elems - 8;
+    cv_voff = ok && !before && !after ? (uint32_t)o * 2u : CV_OUTSIDE;
+    cv_fix[qb] = !ok ? CV_NOFIX
+                     : ((uint32_t)(lo * 9 + hi) * 16u | (before ? (uint32_t)(-o) << 16 : 0u) |
+                        (!before && after ? (uint32_t)(x_elems - o) << 20 : 0u));
+    cv_dst = stage_base;
+    cv_pending = true;
+    int ndw = tap_dw + g.step_dw;
+    const bool wrap_w = ndw >= g.lim_w;
+    ndw -= wrap_w ? g.lim_w : 0;
+    int ndh = tap_dh + g.step_dh + (wrap_w ? g.dil_h : 0);
+    const bool wrap_h = ndh >= g.lim_h;
+    ndh -= wrap_h ? g.lim_h : 0;
+    tap_off += (uint32_t)(g.step_koff + (wrap_w ? g.adj_w : 0) + (wrap_h ? g.adj_h : 0));
+    tap_dw = ndw;
+    tap_dh = ndh;
+  };
+  auto conv_go = [&]() __attribute__((always_inline)) {
+    asm volatile("buffer_load_dwordx4 %0, %1, 0 offen lds" : : "v"(cv_voff), "s"(cv_rsrc) : "memory");
+  };
+  // Fix-up of one op's chunk: zero the elements outside [lo, hi): chunk & mask(lo, hi), the mask read from the
+  // table.  In two parts so that the two LDS reads have returned when the second part runs: fix_read, a few MFMA
+  // slots, fix_write.  Every lane does it for every op, needed or not (its mask is all ones when it has nothing to
+  // zero): straight-line code lets the compiler wait for exactly these reads, where a branch around them made it
+  // wait for every LDS read in flight (measured: 433 with the branch, 618 TFLOP/s with no fix-up at all).
+  // A chunk that could not be fetched whole at either end of the tensor (conv_prepare) was loaded as zeros and
+  // has its inside elements filled in one by one afterwards (fix_special); that happens in a handful of
+  // workgroups at most and costs the others one uniform branch per period.
+  i32x4 cv_rmw[CONV ? C::B_LPW : 1], cv_msk[CONV ? C::B_LPW : 1];
+  auto conv_fix_at = [&](int qb, uint32_t dst) __attribute__((always_inline)) {
+    return dst + C::A_BYTES + (uint32_t)(qb * NW + wave) * 1024u + (uint32_t)lane * 16u;
+  };
+  auto conv_fix_read = [&](int qb, uint32_t note, uint32_t dst) __attribute__((always_inline)) {
+    cv_msk[qb] = *TNX_LDS(i32x4, cv_table + (note & 0xffffu));
+    cv_rmw[qb] = *TNX_LDS(i32x4, conv_fix_at(qb, dst));
+  };
+  auto conv_fix_write = [&](int qb, uint32_t note, uint32_t dst) __attribute__((always_inline)) {
+    *TNX_LDS(i32x4, conv_fix_at(qb, dst)) = cv_rmw[qb] & cv_msk[qb];
+  };
+  auto conv_fix_special = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], uint32_t dst) __attribute__((always_inline)) {
+    uint32_t any = 0;
+#pragma unroll
+    for (int qb = 0; qb < (CONV ? C::B_LPW : 0); ++qb) any |= notes[qb] >> 16;
+    if (__builtin_amdgcn_ballot_w64(any != 0) != 0) {
+#pragma unroll 1
+      for (int qb = 0; qb < (CONV ? C::B_LPW : 0); ++qb) {
+        uint32_t note = 0;
+#pragma unroll
+        for (int x = 0; x < (CONV ? C::B_LPW : 0); ++x) note = x == qb ? notes[x] : note;   // no register-indexed array
+        const int back = (int)((note >> 16) & 0xf), ahead = (int)(note >> 20);
+        if (back || ahead) {
+          const uint32_t at = conv_fix_at(qb, dst);
+          const int idx = (int)((note & 0xffffu) >> 4), lo = idx / 9, hi = idx % 9;
+          const uint16_t* src = (const uint16_t*)p.b + (back ? -back : (int)(p.cv.x_bytes >> 1) - ahead);
+#pragma unroll 1
+          for (int e = lo; e < hi; ++e) *TNX_LDS(uint16_t, at + 2 * e) = src[e];
+        }
+      }
+    }
+  };
+  // the whole fix-up of the slab whose notes are in `notes`, in one go (prologue and the first draining period)
+  auto conv_fixup_all = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], uint32_t dst) __attribute__((always_inline)) {
+    if constexpr (CONV) {
+#pragma unroll
+      for (int qb = 0; qb < C::B_LPW; ++qb) conv_fix_read(qb, notes[qb], dst);
+#pragma unroll
+      for (int qb = 0; qb < C::B_LPW; ++qb) conv_fix_write(qb, notes[qb], dst);
+      conv_fix_special(notes, dst);
+    }
+  };
+  auto conv_fixup = [&]() __attribute__((always_inline)) {
+    if constexpr (CONV) {
+      if (cv_pending) {
+        conv_fixup_all(cv_fix, cv_dst);
+        cv_pending = false;
+      }
+    }
+  };
+  // Inside a period the fix-up works on a copy of the notes taken when the period starts (the period's own B ops
+  // write new notes): part one of op qb behind MFMA slot CV_FS * qb, part two CV_FD slots later.
+  uint32_t cv_old[CONV ? C::B_LPW : 1];
+  uint32_t cv_old_dst = 0;
+  auto conv_period_begin = [&]() __attribute__((always_inline)) {
+    if constexpr (CONV) {
+#pragma unroll
+      for (int qb = 0; qb < C::B_LPW; ++qb) cv_old[qb] = cv_fix[qb];
+      cv_old_dst = cv_dst;
+    }
+  };
+  constexpr int CV_FD = 6;                                                              // slots between read and write
+  constexpr int CV_FS = !CONV ? 1 : ((C::KSTEPS * TM * TN - CV_FD - 1) / C::B_LPW >= 4 ? 4 : 2);
+  static_assert(!CONV || CV_FS * (C::B_LPW - 1) + CV_FD + 1 < C::KSTEPS * TM * TN, "no room for the fix-up in one period");
+  auto conv_fix_slot = [&](int slot) __attribute__((always_inline)) {
+    if constexpr (CONV) {
+#pragma unroll
+      for (int qb = 0; qb < C::B_LPW; ++qb) {
+        if (slot == CV_FS * qb) conv_fix_read(qb, cv_old[qb], cv_old_dst);
+        if (slot == CV_FS * qb + CV_FD) conv_fix_write(qb, cv_old[qb], cv_old_dst);
+      }
+      if (slot == CV_FS * (C::B_LPW - 1) + CV_FD + 1) conv_fix_special(cv_old, cv_old_dst);
+    }
+  };
+
   // one DMA op (q-th of this wave) of local slab t, into ring slot t % STAGES
   auto dma_op = [&](int q, uint32_t stage_base) __attribute__((always_inline)) {
-    if (q < C::A_LPW) {
+    if (CONV && q >= C::A_LPW) {
+      conv_prepare(q - C::A_LPW, stage_base);
+      dma16_set_m0(stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
+      asm volatile("s_nop 0" ::: "memory");
+      conv_go();
+    } else if (q < C::A_LPW) {
       dma16(a_sbase, a_voff[q], stage_base + (q * NW + wave) * 1024);
     } else {
       // short tiles are the ones used on skinny problems, where B is the HBM stream
@@ -865,17 +1192,19 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   };
   // the same op in two parts (see dma16_set_m0): LDS target first, the load after one other instruction
   auto dma_target = [&](int q, uint32_t stage_base) __attribute__((always_inline)) {
+    if (CONV && q >= C::A_LPW) conv_prepare(q - C::A_LPW, stage_base);
     if (q < C::A_LPW) dma16_set_m0(stage_base + (q * NW + wave) * 1024);
     else dma16_set_m0(stage_base + C::A_BYTES + ((q - C::A_LPW) * NW + wave) * 1024);
   };
   auto dma_go = [&](int q) __attribute__((always_inline)) {
-    if (q < C::A_LPW) dma16_go<false>(a_sbase, a_voff[q]);
+    if (CONV && q >= C::A_LPW) conv_go();
+    else if (q < C::A_LPW) dma16_go<false>(a_sbase, a_voff[q]);
     else if (BM <= 64 && p.b_once) dma16_go<true>(b_sbase, b_voff[q - C::A_LPW]);
     else dma16_go<false>(b_sbase, b_voff[q - C::A_LPW]);
   };
   auto dma_advance = [&]() __attribute__((always_inline)) {
     a_sbase += BK * ES;
-    b_sbase += BT ? (int64_t)BK * ES : (int64_t)BK * p.sbk * ES;
+    if (!CONV) b_sbase += BT ? (int64_t)BK * ES : (int64_t)BK * p.sbk * ES;
   };
   auto stage_of = [&](int t) __attribute__((always_inline)) { return lds0 + (uint32_t)(t % STAGES) * C::STAGE_BYTES; };
 
@@ -964,7 +1293,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // longer than it saves; spread further, the last loads are waited for as soon as they are
   // issued), over the first quarter with two waves per SIMD (the other wave covers the stall).
   constexpr int SPAN2 = (NW == 4 ? PERIOD / 2 : PERIOD / 4) > 0 ? (NW == 4 ? PERIOD / 2 : PERIOD / 4) : 1;
-  constexpr int SPAN = (STAGES == 2 || !FAST) ? SPAN2 : PERIOD;
+  // (CONV: three slots, but every load is waited for at the next barrier as with two)
+  constexpr int SPAN = (STAGES == 2 || !FAST || CONV) ? SPAN2 : PERIOD;
+  // loads of this wave that may still be in flight when a period starts (CONV: none, see the kernel's header)
+  constexpr int PWAIT = CONV ? 0 : (STAGES - 2) * C::LPW;
   constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
   constexpr int NEXT0 = C::KSTEPS & 1;                           // set that receives step 0 of the next slab
 
@@ -973,6 +1305,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   auto slot_body = [&](int mset, int x, int rset, int& rd, uint32_t sa, uint32_t sb, int ks_next, bool with_dma, int slot,
                        uint32_t dst) __attribute__((always_inline)) {
     mma_one(mset, x);
+    if (with_dma) conv_fix_slot(slot);
     int lo = 0, hi = 0;
     if (with_dma && slot < SPAN) { lo = slot * C::LPW / SPAN; hi = (slot + 1) * C::LPW / SPAN; }
     const bool paired = hi - lo == 1 && rd < NREAD;
@@ -1025,6 +1358,35 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
 
   // first STAGES slabs of the tile the loader stands on
   auto issue_prologue = [&]() __attribute__((always_inline)) {
+    if constexpr (CONV) {
+      // slabs 0 and 1 are read before any period could fix them: both are issued, waited for and fixed here;
+      // slab 2 is issued afterwards and takes the regular route
+      uint32_t first[C::B_LPW];
+      const uint32_t dst0 = stage_of(0);
+      if (KT > 0) {
+#pragma unroll
+        for (int q = 0; q < C::LPW; ++q) dma_op(q, dst0);
+        dma_advance();
+#pragma unroll
+        for (int qb = 0; qb < C::B_LPW; ++qb) first[qb] = cv_fix[qb];
+      }
+      if (KT > 1) {
+#pragma unroll
+        for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(1));
+        dma_advance();
+      }
+      TNX_WAIT_VM(0);
+      if (KT > 0) conv_fixup_all(first, dst0);
+      if (KT > 1) conv_fixup_all(cv_fix, stage_of(1));
+      cv_pending = false;
+      if (KT > 2) {
+#pragma unroll
+        for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(2));
+        dma_advance();
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the fix-up writes are done before the barrier that follows
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < STAGES; ++s) {
       if (s < KT) {
@@ -1061,9 +1423,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       auto period = [&](auto jtag) __attribute__((always_inline)) {
         constexpr int j = decltype(jtag)::value;
         constexpr int P = (C::KSTEPS & 1) ? (j & 1) : 0;          // parity of the slab whose last k step runs now
-        __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
+        __builtin_amdgcn_s_waitcnt((PWAIT & 0xF) | (((PWAIT >> 4) & 0x3) << 14) | 0x0070);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        conv_period_begin();
         const uint32_t dst = lds0 + (uint32_t)(j % STAGES) * C::STAGE_BYTES;
         const uint32_t sa1 = lds0 + (uint32_t)((j + 1) % STAGES) * C::STAGE_BYTES, sb1 = sa1 + C::A_BYTES;
         last_step(sa1, sb1, Yes{}, dst, IntTag<P>{}, No{});
@@ -1086,9 +1449,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
   }
   for (; t + STAGES < KT; ++t) {
-    __builtin_amdgcn_s_waitcnt((((STAGES - 2) * C::LPW) & 0xF) | (((((STAGES - 2) * C::LPW) >> 4) & 0x3) << 14) | 0x0070);
+    __builtin_amdgcn_s_waitcnt((PWAIT & 0xF) | (((PWAIT >> 4) & 0x3) << 14) | 0x0070);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    conv_period_begin();
     const uint32_t dst = stage_of(t);
     if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
@@ -1106,6 +1470,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     __builtin_amdgcn_s_waitcnt(0x0070);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    conv_fixup();      // CONV: the last slab that was issued has landed; nothing reads it before the next barrier
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
     last_step(sa1, sb1, No{}, 0u, Par0{}, Yes{});
     inner_steps(sa1, sb1, No{}, 0u, Par0{});
@@ -1131,6 +1496,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     const int64_t gm0 = m0 + wy * C::WTM;
     const int64_t gn0 = n0 + wx * C::WTN;
     const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
+    if constexpr (CONV) {
+      epilogue_store_conv<T, C, O>(acc, p.c, strip, lane, (int)gm0, (int)gn0, p.cv);
+      return;
+    }
     if (cut) {
       // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
       const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;

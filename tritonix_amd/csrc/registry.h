@@ -16,6 +16,7 @@ struct KernelEntry {
   launch_fn generic;  // element-wise loader: any strides / ragged k; may be null
   launch_fn persist;  // DMA loader, one workgroup per CU walking its tiles; may be null
   launch_fn fast_bt;  // DMA loader for k-contiguous B (stride_bk == 1, the `x @ w.t()` layout); may be null
+  launch_fn conv;     // conv2d forward on the DMA loader (GemmParams::cv); may be null
 };
 
 // records the hipError_t behind a TNX_E_HIP for tnx_last_hip_error() (per thread)
@@ -26,10 +27,10 @@ struct KernelGroup {
   int count;
 };
 
-template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false>
+template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false, bool CONV = false>
 hipError_t launch_tile(const GemmParams& p, unsigned grid, hipStream_t stream) {
   static_assert(C::VALID, "tile configuration is not buildable");
-  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST, PERSIST, BT>), dim3(grid), dim3(C::THREADS), 0, stream, p);
+  hipLaunchKernelGGL((gemm_tile_kernel<T, C, FAST, PERSIST, BT, CONV>), dim3(grid), dim3(C::THREADS), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -64,10 +65,24 @@ template <class T, class C> struct BtLaunch<T, C, true> {
   static constexpr launch_fn fn = &launch_tile<T, C, true, false, true>;
 };
 
+// The conv2d variant exists for the three-slot, four-wave, 16-bit tiles 128x128, 256x128 and 128x256 with a 128-byte
+// K slab (256x256 has no registers left for the loader's pixel and filter-tap state: it spills inside the K loop).
+template <class C> constexpr bool conv_ok() {
+  return C::ES == 2 && C::NW == 4 && C::STAGES == 3 && C::BK == 64 && C::BM >= 128 && C::BN >= 128 &&
+         C::TM * C::TN * C::ACC_N <= 128;
+}
+template <class T, class C, bool OK = conv_ok<C>()> struct ConvLaunch {
+  static constexpr launch_fn fn = nullptr;
+};
+template <class T, class C> struct ConvLaunch<T, C, true> {
+  static constexpr launch_fn fn = &launch_tile<T, C, true, false, false, true>;
+};
+
 #define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
   {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
    &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \
    GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr,               \
-   PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn, BtLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
+   PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn, BtLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn,     \
+   ConvLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
 
 }  // namespace tnx

@@ -38,6 +38,8 @@ _CANDIDATE_CONFIGS = [
     (256, 128, 64, 8),
 ]
 _CONV_FWD_CONFIG_CACHE: Dict[tuple, dict] = {}
+# optional launch keyword LOADER (no counterpart in the reference): which of the two kernels moves the slabs
+_LOADERS = {"auto": _C.CONV_LOADER_AUTO, "registers": _C.CONV_LOADER_REGISTERS, "dma": _C.CONV_LOADER_DMA}
 
 
 def output_size(h_in: int, w_in: int, filter_h: int, filter_w: int, stride, padding, dilation) -> Tuple[int, int]:
@@ -65,7 +67,7 @@ def _raise_for_status(status: int, a: _C.Conv2dArgs) -> None:
 
 
 def _args(out, input, weight, bias, batch, c_in, h_in, w_in, c_out, filter_h, filter_w, stride, padding, dilation,
-          block_m: int, block_n: int, block_k: int, group_m: int) -> _C.Conv2dArgs:
+          block_m: int, block_n: int, block_k: int, group_m: int, loader: int = 0) -> _C.Conv2dArgs:
     a = _C.Conv2dArgs()
     a.input, a.weight, a.output = input.data_ptr(), weight.data_ptr(), out.data_ptr()
     a.bias = bias.data_ptr() if bias is not None else None
@@ -82,6 +84,7 @@ def _args(out, input, weight, bias, batch, c_in, h_in, w_in, c_out, filter_h, fi
             raise ValueError(f"conv2d_forward: bias dtype {bias.dtype} is not a float type")
         a.bias_dtype = _DTYPES[bias.dtype]
     a.block_pixels, a.block_cout, a.block_k, a.group_pixels = block_m, block_n, block_k, group_m
+    a.loader = loader
     a.stream = torch.cuda.current_stream(input.device).cuda_stream
     return a
 
@@ -142,7 +145,7 @@ class Conv2dForwardKernel:
             raise ValueError("bias must be contiguous")
         return _args(out, x, w, bias, b["BATCH_SIZE"], b["C_IN"], b["H_IN"], b["W_IN"], b["C_OUT"], b["FILTER_H"],
                      b["FILTER_W"], stride, padding, dilation, b["BLOCK_SIZE_M"], b["BLOCK_SIZE_N"], b["BLOCK_SIZE_K"],
-                     b["GROUP_SIZE_M"])
+                     b["GROUP_SIZE_M"], _LOADERS[b.get("LOADER", "auto")])
 
     def run(self, *args, grid=None, **kwargs):
         a = self.bind(*args, **kwargs)
@@ -227,11 +230,11 @@ def conv2d_forward(
                                   "matrix instruction on gfx950")
     out = input.new_empty((n, c_out, h_out, w_out))
 
-    def launch(bm, bn, bk, g, dst=out):
+    def launch(bm, bn, bk, g, loader="auto", dst=out):
         conv2d_forward_kernel[(cdiv(gemm_m, bm), cdiv(gemm_n, bn))](
             dst, input, weight, bias, n, c_in, h_in, w_in, c_out, h_out, w_out, r, s,
             stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], gemm_m, gemm_n, gemm_k,
-            BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=g, USE_TF32=use_tf32)
+            BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=g, USE_TF32=use_tf32, LOADER=loader)
 
     if config is None:
         key = (n, c_in, h_in, w_in, c_out, r, s, stride, padding, dilation, input.dtype)
@@ -250,7 +253,7 @@ def conv2d_forward(
             _CONV_FWD_CONFIG_CACHE[key] = cfg = best
     else:
         cfg = config
-    launch(cfg["BLOCK_SIZE_M"], cfg["BLOCK_SIZE_N"], cfg["BLOCK_SIZE_K"], cfg.get("GROUP_SIZE_M", 8))
+    launch(cfg["BLOCK_SIZE_M"], cfg["BLOCK_SIZE_N"], cfg["BLOCK_SIZE_K"], cfg.get("GROUP_SIZE_M", 8), cfg.get("LOADER", "auto"))
     return out
 
 
