@@ -373,6 +373,19 @@ def headline(torch, dev, oracle, mm, args, operands, out):
     return ok
 
 
+def default_loader(conv_args):
+    """Which of the two conv2d kernels a launch with these arguments runs (tnx_conv_loader), by asking the library."""
+    import ctypes
+
+    from tritonix_amd import _C
+
+    probe = type(conv_args).from_buffer_copy(conv_args)
+    if probe.loader:
+        return probe.loader
+    probe.loader = _C.CONV_LOADER_DMA        # with a tile given, "auto" takes the direct-to-LDS kernel whenever it is allowed
+    return _C.CONV_LOADER_DMA if _C.load().tnx_conv2d_supported(ctypes.byref(probe)) == _C.OK else _C.CONV_LOADER_REGISTERS
+
+
 def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
     res = {}
     reps = 30
@@ -502,35 +515,43 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
         from tritonix_amd.ops.conv2d import conv2d_forward, torch_conv2d_forward
         import tritonix_amd.ops.conv2d.forward as conv
 
-        g = torch.Generator("cpu").manual_seed(66)
-        n_, c_, hw_, k_ = 32, 256, 56, 256
-        x_cpu = torch.randn(n_, c_, hw_, hw_, generator=g).bfloat16()
-        w_cpu = (torch.randn(k_, c_, 3, 3, generator=g) / 48).bfloat16()
-        b_cpu = torch.randn(k_, generator=g).bfloat16()
-        if zeros:
-            x_cpu.zero_(); w_cpu.zero_(); b_cpu.zero_()
-        x, w, b = x_cpu.to(dev), w_cpu.to(dev), b_cpu.to(dev)
-        y = conv2d_forward(x, w, b, (1, 1), (1, 1), (1, 1))          # times the candidate tiles once, as the reference does
-        cfg = next(iter(v for kk, v in conv._CONV_FWD_CONFIG_CACHE.items() if kk[:5] == (n_, c_, hw_, hw_, k_)))
-        flops = 2.0 * n_ * hw_ * hw_ * k_ * c_ * 9
-        bytes_ = 2 * (x.numel() + w.numel() + b.numel() + y.numel())
-        gm, gn, gk = n_ * hw_ * hw_, k_, c_ * 9
-
-        lc = conv.conv2d_forward_kernel.prepare(y, x, w, b, n_, c_, hw_, hw_, k_, hw_, hw_, 3, 3, 1, 1, 1, 1, 1, 1, gm, gn, gk, **cfg)
-        r = measure("CONV", lambda i: lc(), flops, bytes_, "bf16", "mfma")
-        r["tile"] = cfg
-        r["workload"] = "conv2d forward bf16: input [32,256,56,56], weight [256,256,3,3], bias, stride 1, padding 1"
-        ref = oracle.reference_conv2d(x_cpu[5:6], w_cpu, b_cpu, (1, 1), (1, 1), (1, 1))
-        r["parity_ok"] = bool(oracle.within_tolerance(y[5:6], ref)[0])
-        if not args.no_vendor:
-            r["vendor_ms"] = vendor_ms(lambda i: torch_conv2d_forward(x, w, b, (1, 1), (1, 1), (1, 1)))
-            r["vendor_note"] = "torch.nn.functional.conv2d (MIOpen), same tensors"
-        if not args.no_cpu:
-            xf, wf, bf = x_cpu[:2].float(), w_cpu.float(), b_cpu.float()
-            t, n = cpu_time(lambda: torch.nn.functional.conv2d(xf, wf, bf, (1, 1), (1, 1)))
-            r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(flops * 2 / n_ / t / 1e9, 1), "cores": torch.get_num_threads(),
-                        "sample": f"torch fp32 CPU conv2d, first 2 of {n_} images, median of {n}"}
-        del x, w, b, y
+        # name: batch, c_in, h = w, c_out, filter, stride, padding.  CONV is the line quoted; the others show the two
+        # kernels' ranges (small planes, a strided layer that only the register-staged kernel takes)
+        layers = {"CONV": (32, 256, 56, 256, 3, 1, 1), "CONV_128x28": (32, 128, 28, 128, 3, 1, 1),
+                  "CONV_512x14": (32, 512, 14, 512, 3, 1, 1), "CONV_128x56_stride2": (32, 128, 56, 128, 3, 2, 1)}
+        for name, (n_, c_, hw_, k_, f_, st_, pd_) in layers.items():
+            g = torch.Generator("cpu").manual_seed(66)
+            x_cpu = torch.randn(n_, c_, hw_, hw_, generator=g).bfloat16()
+            w_cpu = (torch.randn(k_, c_, f_, f_, generator=g) / (c_ * f_ * f_) ** 0.5).bfloat16()
+            b_cpu = torch.randn(k_, generator=g).bfloat16()
+            if zeros:
+                x_cpu.zero_(); w_cpu.zero_(); b_cpu.zero_()
+            x, w, b = x_cpu.to(dev), w_cpu.to(dev), b_cpu.to(dev)
+            geo = ((st_, st_), (pd_, pd_), (1, 1))
+            y = conv2d_forward(x, w, b, *geo)            # times the candidate tiles once, as the reference does
+            cfg = conv._CONV_FWD_CONFIG_CACHE[(n_, c_, hw_, hw_, k_, f_, f_, *geo, torch.bfloat16)]
+            ho = y.shape[2]
+            flops = 2.0 * n_ * ho * ho * k_ * c_ * f_ * f_
+            bytes_ = 2 * (x.numel() + w.numel() + b.numel() + y.numel())
+            gm, gn, gk = n_ * ho * ho, k_, c_ * f_ * f_
+            lc = conv.conv2d_forward_kernel.prepare(y, x, w, b, n_, c_, hw_, hw_, k_, ho, ho, f_, f_, st_, st_, pd_, pd_, 1, 1,
+                                                    gm, gn, gk, **cfg)
+            r = measure(name, lambda i: lc(), flops, bytes_, "bf16", "mfma")
+            r["tile"] = cfg
+            r["loader"] = {1: "registers", 2: "dma"}[default_loader(lc.args)]
+            r["workload"] = (f"conv2d forward bf16: input [{n_},{c_},{hw_},{hw_}], weight [{k_},{c_},{f_},{f_}], bias, "
+                             f"stride {st_}, padding {pd_}")
+            ref = oracle.reference_conv2d(x_cpu[5:6], w_cpu, b_cpu, *geo)
+            r["parity_ok"] = bool(oracle.within_tolerance(y[5:6], ref)[0])
+            if not args.no_vendor:
+                r["vendor_ms"] = vendor_ms(lambda i: torch_conv2d_forward(x, w, b, *geo))
+                r["vendor_note"] = "torch.nn.functional.conv2d (MIOpen), same tensors"
+            if not args.no_cpu and name == "CONV":
+                xf, wf, bf = x_cpu[:2].float(), w_cpu.float(), b_cpu.float()
+                t, n = cpu_time(lambda: torch.nn.functional.conv2d(xf, wf, bf, *geo))
+                r["cpu"] = {"ms": round(t * 1e3, 3), "gflops": round(flops * 2 / n_ / t / 1e9, 1), "cores": torch.get_num_threads(),
+                            "sample": f"torch fp32 CPU conv2d, first 2 of {n_} images, median of {n}"}
+            del x, w, b, y
 
     # C5: int8 -> int32
     if "C5" in wanted:
