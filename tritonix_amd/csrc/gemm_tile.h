@@ -842,10 +842,10 @@ template <int V> struct IntTag { static constexpr int value = V; };
 // of a chunk that fall into the left / right padding have to be zeroed in LDS afterwards, by the wave that loaded
 // them.  Done between the wait for the loads and the barrier that publishes the slab, that fix-up sits on the
 // critical path of every K slab (measured: 340 instead of 630 TFLOP/s on a 3x3 layer), so the ring has three slots
-// and a slab spends one whole period between landing and being read: slab t+3 is issued during period t, has
-// landed when period t+1 starts (every wave waits for all of its own loads there, as with two slots), is fixed
-// during period t+1 -- one read-modify-write of the chunk per op, slotted behind that period's first MFMAs -- and
-// is published by barrier t+2, before whose period nothing reads it.  16-bit types, stride_w == 1, k % BK == 0.
+// and a slab is fixed well before it is read: slab t+3 is issued during the first half of period t, waited for in
+// the middle of period t+1 (by then only that period's own loads may still be outstanding), fixed in the second
+// half of period t+1 -- one read-modify-write of the chunk per op, slotted behind MFMAs -- and published by barrier
+// t+2, before whose period nothing reads it.  16-bit types, stride_w == 1, k % BK == 0.
 template <class T, class C, bool FAST, bool PERSIST = false, bool BT = false, bool CONV = false>
 __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int ES = C::ES, BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, STAGES = C::STAGES;
@@ -1159,17 +1159,23 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       cv_old_dst = cv_dst;
     }
   };
+  // The period's own loads are all issued in its first half; in the middle of the period the wave waits until only
+  // those are outstanding, i.e. until the slab issued one period earlier has landed (loads retire in issue order),
+  // and fixes that slab in the second half.  A slab so has a period and a half to arrive.
+  constexpr int CV_PERIOD = C::KSTEPS * TM * TN;
+  constexpr int CV_WAIT_SLOT = CV_PERIOD / 2;
   constexpr int CV_FD = 6;                                                              // slots between read and write
-  constexpr int CV_FS = !CONV ? 1 : ((C::KSTEPS * TM * TN - CV_FD - 1) / C::B_LPW >= 4 ? 4 : 2);
-  static_assert(!CONV || CV_FS * (C::B_LPW - 1) + CV_FD + 1 < C::KSTEPS * TM * TN, "no room for the fix-up in one period");
+  constexpr int CV_FS = !CONV ? 1 : ((CV_PERIOD / 2 - CV_FD - 3) / C::B_LPW >= 4 ? 4 : ((CV_PERIOD / 2 - CV_FD - 3) / C::B_LPW >= 2 ? 2 : 1));
+  static_assert(!CONV || CV_WAIT_SLOT + 1 + CV_FS * (C::B_LPW - 1) + CV_FD + 1 < CV_PERIOD, "no room for the fix-up in half a period");
   auto conv_fix_slot = [&](int slot) __attribute__((always_inline)) {
     if constexpr (CONV) {
+      if (slot == CV_WAIT_SLOT) { TNX_WAIT_VM(C::LPW); }
 #pragma unroll
       for (int qb = 0; qb < C::B_LPW; ++qb) {
-        if (slot == CV_FS * qb) conv_fix_read(qb, cv_old[qb], cv_old_dst);
-        if (slot == CV_FS * qb + CV_FD) conv_fix_write(qb, cv_old[qb], cv_old_dst);
+        if (slot == CV_WAIT_SLOT + 1 + CV_FS * qb) conv_fix_read(qb, cv_old[qb], cv_old_dst);
+        if (slot == CV_WAIT_SLOT + 1 + CV_FS * qb + CV_FD) conv_fix_write(qb, cv_old[qb], cv_old_dst);
       }
-      if (slot == CV_FS * (C::B_LPW - 1) + CV_FD + 1) conv_fix_special(cv_old, cv_old_dst);
+      if (slot == CV_WAIT_SLOT + 1 + CV_FS * (C::B_LPW - 1) + CV_FD + 1) conv_fix_special(cv_old, cv_old_dst);
     }
   };
 
@@ -1295,8 +1301,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   constexpr int SPAN2 = (NW == 4 ? PERIOD / 2 : PERIOD / 4) > 0 ? (NW == 4 ? PERIOD / 2 : PERIOD / 4) : 1;
   // (CONV: three slots, but every load is waited for at the next barrier as with two)
   constexpr int SPAN = (STAGES == 2 || !FAST || CONV) ? SPAN2 : PERIOD;
-  // loads of this wave that may still be in flight when a period starts (CONV: none, see the kernel's header)
-  constexpr int PWAIT = CONV ? 0 : (STAGES - 2) * C::LPW;
+  // loads of this wave that may still be in flight when a period starts (CONV: the slab issued in the period
+  // before, which is waited for in the middle of this one)
+  constexpr int PWAIT = CONV ? C::LPW : (STAGES - 2) * C::LPW;
   constexpr int LAST = (C::KSTEPS - 1) & 1;                      // register set holding the last k step
   constexpr int NEXT0 = C::KSTEPS & 1;                           // set that receives step 0 of the next slab
 
