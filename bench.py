@@ -444,6 +444,16 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
         if not args.no_vendor:
             cv = torch.empty_like(c)
             r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, bs[i % nrot], out=cv), reps=reps)
+            # what plain streaming kernels of the vendor's library reach on the same rotating copies of B: a read-only
+            # reduction and a copy (read + write), as context for a fraction of the nominal 8 TB/s
+            flat = [t.view(-1).view(torch.float32) for t in bs]       # (bit patterns of bf16 pairs: all finite or not, the traffic is the same)
+            sink = torch.empty_like(flat[0])
+            t_sum = vendor_ms(lambda i: flat[i % nrot].max(), reps=reps)
+            t_cp = vendor_ms(lambda i: sink.copy_(flat[i % nrot]), reps=reps)
+            nb = flat[0].numel() * 4
+            r["vendor_stream"] = {"max_read_gbs": round(nb / t_sum / 1e6, 1), "copy_read_plus_write_gbs": round(2 * nb / t_cp / 1e6, 1),
+                                  "bytes": nb}
+            del flat, sink
         if not args.no_cpu:
             af, bf = a_cpu.float(), b_cpu.float()
             t, n = cpu_time(lambda: torch.matmul(af, bf))
