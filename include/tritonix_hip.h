@@ -233,7 +233,8 @@ int tnx_conv2d_supported(const tnx_conv2d_args* args);
  * back <= 0 for a filter larger than the padded image, which tnx_conv2d_forward rejects. */
 void tnx_conv2d_output_size(const tnx_conv2d_args* args, int32_t* h_out, int32_t* w_out);
 
-/* Fill block_pixels / block_cout / block_k / group_pixels with the built-in choice for this problem. */
+/* Fill block_pixels / block_cout / block_k / group_pixels / loader with the built-in choice for this problem (a
+ * non-NULL weight pointer is checked for the 16-byte alignment the direct-to-LDS kernel needs). */
 int tnx_conv2d_default_config(tnx_conv2d_args* args);
 
 /* Compiled conv2d tiles: count, and "dtype block_cout block_pixels block_k loader" of the i-th (static storage;

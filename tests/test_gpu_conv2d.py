@@ -109,6 +109,35 @@ def test_loader_that_does_not_fit_is_refused(device):
     assert oracle.within_tolerance(out, _oracle(x, wt, None, stride, padding, dilation))[0]
 
 
+def test_weight_that_is_not_16_byte_aligned_takes_the_register_kernel(device):
+    x, wt, b, stride, padding, dilation = _inputs(DMA_CASES["3x3_same"], torch.bfloat16, seed=2)
+    store = torch.empty(wt.numel() + 1, dtype=wt.dtype, device=device)
+    wd = store[1:].view(wt.shape)                       # 2 bytes past a 16-byte boundary
+    wd.copy_(wt)
+    assert wd.data_ptr() % 16 == 2 and wd.is_contiguous()
+    ref = _oracle(x, wt, b, stride, padding, dilation)
+    cfg = dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64)
+    out = conv2d_forward(x.to(device), wd, b.to(device), stride, padding, dilation, config=cfg)
+    assert oracle.within_tolerance(out, ref)[0]
+    with pytest.raises(ValueError):
+        conv2d_forward(x.to(device), wd, b.to(device), stride, padding, dilation, config=dict(cfg, LOADER="dma"))
+    # an input that is only 2-byte aligned is fine for both kernels
+    xs = torch.empty(x.numel() + 1, dtype=x.dtype, device=device)
+    xd = xs[1:].view(x.shape)
+    xd.copy_(x)
+    out = conv2d_forward(xd, wt.to(device), b.to(device), stride, padding, dilation, config=dict(cfg, LOADER="dma"))
+    assert oracle.within_tolerance(out, ref)[0]
+    # so is an output that is only 2-byte aligned (the epilogue's 16-byte stores take any element address)
+    ys = torch.empty(ref.numel() + 1, dtype=x.dtype, device=device)
+    yd = ys[1:].view(ref.shape)
+    n, c, h, w = x.shape
+    k, _, r, s_ = wt.shape
+    conv2d_forward_kernel[(1,)](yd, xd, wt.to(device), b.to(device), n, c, h, w, k, ref.shape[2], ref.shape[3], r, s_, stride[0],
+                                stride[1], padding[0], padding[1], dilation[0], dilation[1], n * ref.shape[2] * ref.shape[3], k,
+                                c * r * s_, BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, GROUP_SIZE_M=8, LOADER="dma")
+    assert oracle.within_tolerance(yd, ref)[0]
+
+
 def test_float32_bias_and_no_bias_agree_with_the_oracle(device):
     x, wt, _, stride, padding, dilation = _inputs(CASES["3x3_same"], torch.bfloat16, seed=3)
     b32 = torch.randn(wt.shape[0], generator=torch.Generator().manual_seed(4))

@@ -257,7 +257,7 @@ extern "C" int tnx_conv2d_default_config(tnx_conv2d_args* a) {
   tnx_conv2d_args tmp = *a;
   tmp.block_cout = tmp.block_pixels = tmp.block_k = 0;
   Resolved r;
-  const int st = resolve(&tmp, &r, false);
+  const int st = resolve(&tmp, &r, a->weight != nullptr);     // a weight pointer, when given, is checked for alignment
   if (st != TNX_OK) return st;
   a->block_cout = r.bcout;
   a->block_pixels = r.bpix;
