@@ -94,6 +94,40 @@ def test_direct_to_lds_loader_matches_the_oracle_and_the_register_kernel(name, d
         assert torch.equal(out, regs), (name, dtype, cfg)
 
 
+def test_seeded_random_geometries_on_both_kernels(device):
+    """Sixty geometries drawn from a fixed seed (filters 1-5 per side, dilation 1-3, padding 0-4, stride_h 1-3, planes
+    3-40 wide, 64 or 128 input channels so that the direct-to-LDS kernel applies): the register-staged kernel against
+    the CPU library routine in fp32, and the direct-to-LDS kernel bit for bit against the register-staged one."""
+    rng = np.random.default_rng(2024)
+    done = 0
+    while done < 60:
+        r, s_ = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        dil = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pad = (int(rng.integers(0, 5)), int(rng.integers(0, 5)))
+        stride = (int(rng.integers(1, 4)), 1)
+        h, w = int(rng.integers(3, 41)), int(rng.integers(3, 41))
+        c_in = int(rng.choice([64, 128]))
+        c_out = int(rng.integers(1, 300))
+        n = int(rng.integers(1, 4))
+        ho, wo = conv.output_size(h, w, r, s_, stride, pad, dil)
+        if ho <= 0 or wo <= 0 or (c_in * r * s_) % 64:
+            continue
+        done += 1
+        g = torch.Generator().manual_seed(done)
+        x = torch.randn(n, c_in, h, w, generator=g).bfloat16()
+        wt = (torch.randn(c_out, c_in, r, s_, generator=g) / (c_in * r * s_) ** 0.5).bfloat16()
+        b = torch.randn(c_out, generator=g).bfloat16() if done % 2 else None
+        xd, wd, bd = x.to(device), wt.to(device), None if b is None else b.to(device)
+        tile = [(128, 128), (128, 256), (256, 128)][done % 3]
+        regs = conv2d_forward(xd, wd, bd, stride, pad, dil,
+                              config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64, LOADER="registers"))
+        dma = conv2d_forward(xd, wd, bd, stride, pad, dil,
+                             config=dict(BLOCK_SIZE_M=tile[0], BLOCK_SIZE_N=tile[1], BLOCK_SIZE_K=64, LOADER="dma"))
+        what = (done, n, c_in, h, w, c_out, r, s_, stride, pad, dil, tile)
+        assert oracle.within_tolerance(regs, oracle.reference_conv2d(x, wt, b, stride, pad, dil))[0], what
+        assert torch.equal(dma, regs), what
+
+
 def test_loader_that_does_not_fit_is_refused(device):
     x, wt, b, stride, padding, dilation = _inputs(CASES["1x1_stride2"], torch.bfloat16)
     with pytest.raises(ValueError):           # stride_w == 2
