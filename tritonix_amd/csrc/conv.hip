@@ -13,16 +13,23 @@ using namespace tnx;
 extern "C" const ConvGroup* tnx_conv_groups(int* ngroups);      // generated
 extern "C" const KernelGroup* tnx_kernel_groups(int* ngroups);  // generated
 
-// the GEMM kernel's conv2d variant for this tile (four waves, three ring slots), or null
+// The GEMM kernel's conv2d variant for this tile (three ring slots), or null.  Built with four and with eight waves;
+// eight are taken when built: the loader's address arithmetic and the fix-up are vector instructions in the MFMA
+// stream, and with two waves per SIMD one wave's arithmetic runs under the other's MFMAs (measured on 3x3 layers,
+// batch 32: 256x128 524 -> 620 TFLOP/s at 56x56 / 256 channels, 128x128 248 -> 292 at 28x28 / 128 and 351 -> 420 at
+// 14x14 / 512).
 static const KernelEntry* find_dma(int dtype, int bcout, int bpix, int bk) {
   int ng = 0;
   const KernelGroup* g = tnx_kernel_groups(&ng);
+  const KernelEntry* four = nullptr;
   for (int i = 0; i < ng; ++i)
     for (int j = 0; j < g[i].count; ++j) {
       const KernelEntry& e = g[i].entries[j];
-      if (e.dtype == dtype && e.bm == bcout && e.bn == bpix && e.bk == bk && e.nw == 4 && e.stages == 3 && e.conv) return &e;
+      if (e.dtype != dtype || e.bm != bcout || e.bn != bpix || e.bk != bk || e.stages != 3 || !e.conv) continue;
+      if (e.nw == 8) return &e;
+      if (e.nw == 4) four = &e;
     }
-  return nullptr;
+  return four;
 }
 
 static const ConvEntry* find_conv(int dtype, int bcout, int bpix, int bk) {
@@ -240,7 +247,7 @@ static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p,
   g.div_s = make_fastdiv((uint32_t)g.fw);
   g.dil_h = a->dil_h; g.dil_w = a->dil_w;
   // k rows one DMA op of the workgroup covers: 256 lanes x 16 bytes over rows of block_pixels * 2 bytes
-  const int rows_per_op = 4 * 64 / (r.bpix * 2 / 16);
+  const int rows_per_op = r.dma->nw * 64 / (r.bpix * 2 / 16);
   tap_step(a, rows_per_op, g.hw_in, &g.step_dw, &g.step_dh, &g.step_koff, &g.lim_w, &g.lim_h, &g.adj_w, &g.adj_h);
   g.bias = (const uint8_t*)a->bias;
   g.bias_dtype = a->bias_dtype;
@@ -302,7 +309,8 @@ template <class F> static void each_conv_kernel(F f) {
   const KernelGroup* k = tnx_kernel_groups(&ng);
   for (int i = 0; i < ng; ++i)
     for (int j = 0; j < k[i].count; ++j)
-      if (k[i].entries[j].conv) f(k[i].entries[j].dtype, k[i].entries[j].bm, k[i].entries[j].bn, k[i].entries[j].bk, true);
+      if (k[i].entries[j].conv && find_dma(k[i].entries[j].dtype, k[i].entries[j].bm, k[i].entries[j].bn, k[i].entries[j].bk) == &k[i].entries[j])
+        f(k[i].entries[j].dtype, k[i].entries[j].bm, k[i].entries[j].bn, k[i].entries[j].bk, true);
 }
 
 extern "C" int tnx_conv2d_kernel_count(void) {

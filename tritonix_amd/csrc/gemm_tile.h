@@ -1164,7 +1164,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // and fixes that slab in the second half.  A slab so has a period and a half to arrive.
   constexpr int CV_PERIOD = C::KSTEPS * TM * TN;
   constexpr int CV_WAIT_SLOT = CV_PERIOD / 2;
-  constexpr int CV_FD = 6;                                                              // slots between read and write
+  constexpr int CV_FD = CV_PERIOD >= 32 ? 6 : 3;                                        // slots between read and write
   constexpr int CV_FS = !CONV ? 1 : ((CV_PERIOD / 2 - CV_FD - 3) / C::B_LPW >= 4 ? 4 : ((CV_PERIOD / 2 - CV_FD - 3) / C::B_LPW >= 2 ? 2 : 1));
   static_assert(!CONV || CV_WAIT_SLOT + 1 + CV_FS * (C::B_LPW - 1) + CV_FD + 1 < CV_PERIOD, "no room for the fix-up in half a period");
   auto conv_fix_slot = [&](int slot) __attribute__((always_inline)) {
