@@ -68,9 +68,9 @@ static void builtin_tile(const tnx_conv2d_args* a, int64_t pixels, int* bcout, i
 }
 
 // Direct-to-LDS kernel: 256 channels x 128 pixels when that still leaves every CU two tiles, else 128 x 128.
-// Measured on 3x3 layers (batch 32): 256x128 538 against 389 TFLOP/s for 128x128 at 56x56 / 256 channels, 128x128
-// ahead of it at 28x28 / 128 channels (244 : 181) and 14x14 / 512 channels (352 : 282), and both well ahead of
-// the register-staged kernel (392, 162, 165) down to a few dozen tiles.
+// Measured on 3x3 layers (batch 32, eight-wave builds): 256x128 620 against 476 TFLOP/s for 128x128 at 56x56 / 256
+// channels, 128x128 ahead of it at 28x28 / 128 channels (292 : 228) and 14x14 / 512 channels (420 : 337), and both
+// well ahead of the register-staged kernel (392, 162, 165) down to a few dozen tiles.
 static bool builtin_dma_tile(const tnx_conv2d_args* a, int h_out, int w_out, int* bcout, int* bpix, int* bk) {
   const int64_t cols = (int64_t)a->batch * h_out * ((w_out + 7) / 8 * 8);
   const int64_t t256 = ((cols + 127) / 128) * (((int64_t)a->c_out + 255) / 256);
@@ -95,7 +95,9 @@ static void tap_step(const tnx_conv2d_args* a, int rows, int hw_in, int* step_dw
   const int sc = rows / rs, sh = (rows % rs) / a->filter_w, sw = rows % a->filter_w;
   *step_dw = sw * a->dil_w;
   *step_dh = sh * a->dil_h;
-  *step_koff = sc * hw_in + *step_dh * a->w_in + *step_dw;
+  // (unsigned: for planes so large that `rows` channels further leaves the tensor the sum may wrap; such taps are
+  // past the last k and never used)
+  *step_koff = (int)((uint32_t)sc * (uint32_t)hw_in + (uint32_t)(*step_dh * a->w_in + *step_dw));
   *lim_w = a->filter_w * a->dil_w;
   *lim_h = a->filter_h * a->dil_h;
   *adj_w = a->dil_h * a->w_in - *lim_w;          // dw wraps: one filter row down
