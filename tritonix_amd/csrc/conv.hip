@@ -248,9 +248,8 @@ static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p,
   g.div_rs = make_fastdiv((uint32_t)g.rs);
   g.div_s = make_fastdiv((uint32_t)g.fw);
   g.dil_h = a->dil_h; g.dil_w = a->dil_w;
-  // k rows one DMA op of the workgroup covers: 256 lanes x 16 bytes over rows of block_pixels * 2 bytes
-  const int rows_per_op = r.dma->nw * 64 / (r.bpix * 2 / 16);
-  tap_step(a, rows_per_op, g.hw_in, &g.step_dw, &g.step_dh, &g.step_koff, &g.lim_w, &g.lim_h, &g.adj_w, &g.adj_h);
+  // the taps are tabulated slab by slab: one step is block_k rows
+  tap_step(a, r.bk, g.hw_in, &g.step_dw, &g.step_dh, &g.step_koff, &g.lim_w, &g.lim_h, &g.adj_w, &g.adj_h);
   g.bias = (const uint8_t*)a->bias;
   g.bias_dtype = a->bias_dtype;
   *grid = (unsigned)((int64_t)p->tiles_m * p->tiles_n);

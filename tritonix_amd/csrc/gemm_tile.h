@@ -70,8 +70,8 @@ struct ConvGeom {
   FastDiv div_hwp, div_wp;         // by h_out*wp, by wp
   FastDiv div_rs, div_s;           // by R*S, by S
   int rs, fw, dil_h, dil_w;
-  // one DMA op further along k (the rows one op of the workgroup covers): what is added to a tap's (dw, dh, element
-  // offset), the limits at which dw and dh wrap, and what a wrap adds to the element offset
+  // one K slab (block_k rows) further along k: what is added to a tap's (dw, dh, element offset), the limits at which
+  // dw and dh wrap, and what a wrap adds to the element offset
   int step_dw, step_dh, step_koff, lim_w, lim_h, adj_w, adj_h;
   const uint8_t* bias;             // [c_out] or null
   int bias_dtype;
@@ -862,8 +862,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // one workgroup per tile: the epilogue strips are laid over the ring once the K loop is done.
   // persistent: the ring is refilled for the next tile during the epilogue, so the strips follow it.
   constexpr int RING_OR_STRIPS = C::LDS_BYTES > EpiStage<C>::BYTES ? C::LDS_BYTES : EpiStage<C>::BYTES;
-  // CONV: behind the ring, a table of the 81 16-byte masks that keep elements [lo, hi) of a chunk (0 <= lo, hi <= 8)
-  constexpr int CV_TABLE_BYTES = CONV ? 81 * 16 : 0;
+  // CONV: behind the ring, a table of the 81 16-byte masks that keep elements [lo, hi) of a chunk (0 <= lo, hi <= 8),
+  // and two tables of the filter taps of one K slab (BK entries of 8 bytes: element offset, dh | dw << 16)
+  constexpr int CV_TABLE_BYTES = CONV ? 81 * 16 + 2 * BK * 8 : 0;
   constexpr int SMEM_BYTES = (PERSIST ? C::LDS_BYTES + PairStrip<C>::BYTES : RING_OR_STRIPS) + CV_TABLE_BYTES;
   static_assert(SMEM_BYTES <= 163840, "LDS budget of one CU exceeded");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[SMEM_BYTES];
@@ -924,18 +925,24 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // CONV: a lane's B ops all fetch the same 16-byte LDS column slot; the pixel chunk that lands there is one of
   // two (the LDS swizzle moves it by two chunks depending on the k row): element offset of (image, channel 0,
   // h0, w0) and the packed (h0, w0) for both, (h0, w0) being the input position of filter tap (0, 0).  Pixels past
-  // the end get h0 = -32768, which no tap brings back into the image.  One running filter tap per lane, advanced
-  // after every op by the k rows the workgroup covers per op (additions and wrap-arounds only).
+  // the end get h0 = -32768, which no tap brings back into the image.  The filter taps (dh, dw, element offset) of
+  // the k rows of a slab come from a 64-entry table in LDS that the first 64 threads write one period ahead, each
+  // keeping the running tap of one k row and moving it one slab on per period (additions and wrap-arounds only):
+  // per op a lane reads one entry instead of doing that arithmetic itself.
   constexpr int CONV_STEP = (NW * 64) / C::CPR_B;          // k rows covered by one B op of the workgroup
   const int cv_r0 = tid / C::CPR_B;                          // k row of this lane in the first op of a slab
   int pix_off0 = 0, pix_off1 = 0, pix_hw0 = 0, pix_hw1 = 0;   // (scalars, not arrays: an array indexed by a run-time bit is moved to LDS by the compiler)
-  int tap_dh = 0, tap_dw = 0;
+  int tap_dh = 0, tap_dw = 0;                                // (wave 0 only) tap of k row `tid` of the next slab to tabulate
   uint32_t tap_off = 0;
+  int cv_wr = 0, cv_rd = 0;                                  // next slab to tabulate / to issue (their parities pick the table)
+  i32x2 cv_ent[CONV ? C::B_LPW : 1];                         // the table entries of this lane's ops of the slab being issued
   uint32_t cv_fix[CONV ? C::B_LPW : 1];                      // per op of the slab in flight: what its fix-up has to do
+  int cv_o[CONV ? C::B_LPW : 1];                             // ... and the element offset its chunk starts at
   bool cv_pending = false;
   uint32_t cv_dst = 0;
   constexpr uint32_t CV_OUTSIDE = 0xffffffffu, CV_NOFIX = 8u * 16u;   // a note is the byte offset of mask (lo, hi) in the table: (lo * 9 + hi) * 16
   const uint32_t cv_table = lds0 + RING_OR_STRIPS;
+  const uint32_t cv_ktab = cv_table + 81 * 16;
   i32x4 cv_rsrc = {0, 0, 0, 0};
   if constexpr (CONV) {
     if (tid < 81) {
@@ -989,13 +996,16 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
           const int hw = (int)(((uint32_t)h0 << 16) | ((uint32_t)w0 & 0xffffu));
           if (v == 0) { pix_off0 = off; pix_hw0 = hw; } else { pix_off1 = off; pix_hw1 = hw; }
         }
-        // the tap of k row cv_r0 (the K loop starts at k = 0: these kernels are never cut along K)
-        const int cin = (int)fd_div((uint32_t)cv_r0, g.div_rs);
-        const int r = cv_r0 - cin * g.rs;
+        // the tap of k row tid (< BK) of slab 0 (the K loop starts at k = 0: these kernels are never cut along K)
+        const int krow = tid & (BK - 1);
+        const int cin = (int)fd_div((uint32_t)krow, g.div_rs);
+        const int r = krow - cin * g.rs;
         const int th = (int)fd_div((uint32_t)r, g.div_s);
         tap_dh = th * g.dil_h;
         tap_dw = (r - th * g.fw) * g.dil_w;
         tap_off = (uint32_t)(cin * g.hw_in + tap_dh * g.w_in + tap_dw);
+        cv_wr = 0;
+        cv_rd = 0;
       }
       const int64_t nrem = p.n - 1 - n0;  // last valid column inside this tile
 #pragma unroll
@@ -1052,7 +1062,36 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
   };
 
-  // CONV: byte offset of B op qb's chunk inside the input (or CV_OUTSIDE), its fix-up note, and the tap moved on
+  // CONV: the first 64 threads write the taps of the next slab to tabulate into the table of its parity and move
+  // their tap one slab on; every lane reads the entries of its ops of the slab that is about to be issued.
+  auto conv_tab_write = [&]() __attribute__((always_inline)) {
+    if constexpr (CONV) {
+      const ConvGeom& g = p.cv;
+      if (wave == 0) {
+        *TNX_LDS(i32x2, cv_ktab + (uint32_t)(cv_wr & 1) * (BK * 8) + (uint32_t)lane * 8u) =
+            i32x2{(int)tap_off, (int)((uint32_t)tap_dh | ((uint32_t)tap_dw << 16))};
+        int ndw = tap_dw + g.step_dw;
+        const bool wrap_w = ndw >= g.lim_w;
+        ndw -= wrap_w ? g.lim_w : 0;
+        int ndh = tap_dh + g.step_dh + (wrap_w ? g.dil_h : 0);
+        const bool wrap_h = ndh >= g.lim_h;
+        ndh -= wrap_h ? g.lim_h : 0;
+        tap_off += (uint32_t)(g.step_koff + (wrap_w ? g.adj_w : 0) + (wrap_h ? g.adj_h : 0));
+        tap_dw = ndw;
+        tap_dh = ndh;
+      }
+      ++cv_wr;
+    }
+  };
+  auto conv_tab_read = [&]() __attribute__((always_inline)) {
+    if constexpr (CONV) {
+#pragma unroll
+      for (int qb = 0; qb < C::B_LPW; ++qb)
+        cv_ent[qb] = *TNX_LDS(i32x2, cv_ktab + (uint32_t)(cv_rd & 1) * (BK * 8) + (uint32_t)(qb * CONV_STEP + cv_r0) * 8u);
+      ++cv_rd;
+    }
+  };
+  // CONV: byte offset of B op qb's chunk inside the input (or CV_OUTSIDE) and its fix-up note
   uint32_t cv_voff = 0;
   auto conv_prepare = [&](int qb, uint32_t stage_base) __attribute__((always_inline)) {
     const ConvGeom& g = p.cv;
@@ -1060,32 +1099,21 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     const bool second = ((row >> 3) ^ (row >> 4)) & 1;      // the pass term of swzB
     const int off = second ? pix_off1 : pix_off0, hw = second ? pix_hw1 : pix_hw0;
     const int h0 = hw >> 16, w0 = (int)(int16_t)(hw & 0xffff);
-    const int o = off + (int)tap_off;
-    int lo = -(w0 + tap_dw), hi = g.w_in - (w0 + tap_dw);    // elements [lo, hi) of the chunk lie inside the input row
+    const int dh = cv_ent[qb].y & 0xffff, dw = (int)((uint32_t)cv_ent[qb].y >> 16);
+    const int o = off + cv_ent[qb].x;
+    int lo = -(w0 + dw), hi = g.w_in - (w0 + dw);            // elements [lo, hi) of the chunk lie inside the input row
     lo = lo < 0 ? 0 : lo;
     hi = hi > 8 ? 8 : hi;
-    const bool ok = (uint32_t)(h0 + tap_dh) < (uint32_t)g.h_in && lo < hi;
+    const bool ok = (uint32_t)(h0 + dh) < (uint32_t)g.h_in && lo < hi;
     // A chunk that starts before the tensor (first row of the first image, left padding) or ends after it (last
-    // row of the last image, right padding) cannot be fetched whole -- the buffer bound drops every dword that is
-    // not entirely inside, valid elements included: it is loaded as zeros and its inside elements are written by
-    // the fix-up.  -o resp. (elements - o) is below 8 in those cases and is all the fix-up needs to find them.
-    const int x_elems = (int)(g.x_bytes >> 1);
-    const bool before = o < 0, after = o > x_elems - 8;
-    cv_voff = ok && !before && !after ? (uint32_t)o * 2u : CV_OUTSIDE;
-    cv_fix[qb] = !ok ? CV_NOFIX
-                     : ((uint32_t)(lo * 9 + hi) * 16u | (before ? (uint32_t)(-o) << 16 : 0u) |
-                        (!before && after ? (uint32_t)(x_elems - o) << 20 : 0u));
+    // row of the last image, right padding) cannot be fetched whole: the buffer bound drops every dword that is not
+    // entirely inside, valid elements included (a negative offset wraps to one past every bound).  Its inside
+    // elements are written by the fix-up, which recognises the case from the offset kept here.
+    cv_voff = ok ? (uint32_t)o * 2u : CV_OUTSIDE;
+    cv_fix[qb] = ok ? (uint32_t)(lo * 9 + hi) * 16u : CV_NOFIX;
+    cv_o[qb] = o;
     cv_dst = stage_base;
     cv_pending = true;
-    int ndw = tap_dw + g.step_dw;
-    const bool wrap_w = ndw >= g.lim_w;
-    ndw -= wrap_w ? g.lim_w : 0;
-    int ndh = tap_dh + g.step_dh + (wrap_w ? g.dil_h : 0);
-    const bool wrap_h = ndh >= g.lim_h;
-    ndh -= wrap_h ? g.lim_h : 0;
-    tap_off += (uint32_t)(g.step_koff + (wrap_w ? g.adj_w : 0) + (wrap_h ? g.adj_h : 0));
-    tap_dw = ndw;
-    tap_dh = ndh;
   };
   auto conv_go = [&]() __attribute__((always_inline)) {
     asm volatile("buffer_load_dwordx4 %0, %1, 0 offen lds" : : "v"(cv_voff), "s"(cv_rsrc) : "memory");
@@ -1109,21 +1137,26 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   auto conv_fix_write = [&](int qb, uint32_t note, uint32_t dst) __attribute__((always_inline)) {
     *TNX_LDS(i32x4, conv_fix_at(qb, dst)) = cv_rmw[qb] & cv_msk[qb];
   };
-  auto conv_fix_special = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], uint32_t dst) __attribute__((always_inline)) {
-    uint32_t any = 0;
+  auto conv_fix_special = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], const int (&os)[CONV ? C::B_LPW : 1],
+                              uint32_t dst) __attribute__((always_inline)) {
+    const int x_elems = (int)(p.cv.x_bytes >> 1);
+    bool any = false;
 #pragma unroll
-    for (int qb = 0; qb < (CONV ? C::B_LPW : 0); ++qb) any |= notes[qb] >> 16;
-    if (__builtin_amdgcn_ballot_w64(any != 0) != 0) {
+    for (int qb = 0; qb < (CONV ? C::B_LPW : 0); ++qb) any |= notes[qb] != CV_NOFIX && (os[qb] < 0 || os[qb] > x_elems - 8);
+    if (__builtin_amdgcn_ballot_w64(any) != 0) {
 #pragma unroll 1
       for (int qb = 0; qb < (CONV ? C::B_LPW : 0); ++qb) {
-        uint32_t note = 0;
+        uint32_t note = CV_NOFIX;
+        int o = 0;
 #pragma unroll
-        for (int x = 0; x < (CONV ? C::B_LPW : 0); ++x) note = x == qb ? notes[x] : note;   // no register-indexed array
-        const int back = (int)((note >> 16) & 0xf), ahead = (int)(note >> 20);
-        if (back || ahead) {
+        for (int x = 0; x < (CONV ? C::B_LPW : 0); ++x) {   // no register-indexed array
+          note = x == qb ? notes[x] : note;
+          o = x == qb ? os[x] : o;
+        }
+        if (note != CV_NOFIX && (o < 0 || o > x_elems - 8)) {
           const uint32_t at = conv_fix_at(qb, dst);
-          const int idx = (int)((note & 0xffffu) >> 4), lo = idx / 9, hi = idx % 9;
-          const uint16_t* src = (const uint16_t*)p.b + (back ? -back : (int)(p.cv.x_bytes >> 1) - ahead);
+          const int idx = (int)(note >> 4), lo = idx / 9, hi = idx % 9;
+          const uint16_t* src = (const uint16_t*)p.b + o;
 #pragma unroll 1
           for (int e = lo; e < hi; ++e) *TNX_LDS(uint16_t, at + 2 * e) = src[e];
         }
@@ -1131,19 +1164,20 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
   };
   // the whole fix-up of the slab whose notes are in `notes`, in one go (prologue and the first draining period)
-  auto conv_fixup_all = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], uint32_t dst) __attribute__((always_inline)) {
+  auto conv_fixup_all = [&](const uint32_t (&notes)[CONV ? C::B_LPW : 1], const int (&os)[CONV ? C::B_LPW : 1],
+                            uint32_t dst) __attribute__((always_inline)) {
     if constexpr (CONV) {
 #pragma unroll
       for (int qb = 0; qb < C::B_LPW; ++qb) conv_fix_read(qb, notes[qb], dst);
 #pragma unroll
       for (int qb = 0; qb < C::B_LPW; ++qb) conv_fix_write(qb, notes[qb], dst);
-      conv_fix_special(notes, dst);
+      conv_fix_special(notes, os, dst);
     }
   };
   auto conv_fixup = [&]() __attribute__((always_inline)) {
     if constexpr (CONV) {
       if (cv_pending) {
-        conv_fixup_all(cv_fix, cv_dst);
+        conv_fixup_all(cv_fix, cv_o, cv_dst);
         cv_pending = false;
       }
     }
@@ -1151,12 +1185,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // Inside a period the fix-up works on a copy of the notes taken when the period starts (the period's own B ops
   // write new notes): part one of op qb behind MFMA slot CV_FS * qb, part two CV_FD slots later.
   uint32_t cv_old[CONV ? C::B_LPW : 1];
+  int cv_old_o[CONV ? C::B_LPW : 1];
   uint32_t cv_old_dst = 0;
+  // ... and the lanes fetch the table entries of the slab this period issues, and the first 64 threads tabulate the
+  // slab after it (into the table that was last read one period ago, before the barrier that has just been passed)
   auto conv_period_begin = [&]() __attribute__((always_inline)) {
     if constexpr (CONV) {
 #pragma unroll
-      for (int qb = 0; qb < C::B_LPW; ++qb) cv_old[qb] = cv_fix[qb];
+      for (int qb = 0; qb < C::B_LPW; ++qb) { cv_old[qb] = cv_fix[qb]; cv_old_o[qb] = cv_o[qb]; }
       cv_old_dst = cv_dst;
+      conv_tab_read();
+      conv_tab_write();
     }
   };
   // The period's own loads are all issued in its first half; in the middle of the period the wave waits until only
@@ -1175,7 +1214,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         if (slot == CV_WAIT_SLOT + 1 + CV_FS * qb) conv_fix_read(qb, cv_old[qb], cv_old_dst);
         if (slot == CV_WAIT_SLOT + 1 + CV_FS * qb + CV_FD) conv_fix_write(qb, cv_old[qb], cv_old_dst);
       }
-      if (slot == CV_WAIT_SLOT + 1 + CV_FS * (C::B_LPW - 1) + CV_FD + 1) conv_fix_special(cv_old, cv_old_dst);
+      if (slot == CV_WAIT_SLOT + 1 + CV_FS * (C::B_LPW - 1) + CV_FD + 1) conv_fix_special(cv_old, cv_old_o, cv_old_dst);
     }
   };
 
@@ -1367,30 +1406,43 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   auto issue_prologue = [&]() __attribute__((always_inline)) {
     if constexpr (CONV) {
       // slabs 0 and 1 are read before any period could fix them: both are issued, waited for and fixed here;
-      // slab 2 is issued afterwards and takes the regular route
+      // slab 2 is issued afterwards and takes the regular route.  The tap tables of slabs 0..3 are written on the
+      // way, each behind a barrier that separates it from the reads of the table it replaces; the table of slab 3
+      // is published by the first period's barrier.
       uint32_t first[C::B_LPW];
+      int first_o[C::B_LPW];
       const uint32_t dst0 = stage_of(0);
+      conv_tab_write();                       // slab 0 -> table 0
+      __syncthreads();
+      conv_tab_read();
       if (KT > 0) {
 #pragma unroll
         for (int q = 0; q < C::LPW; ++q) dma_op(q, dst0);
         dma_advance();
 #pragma unroll
-        for (int qb = 0; qb < C::B_LPW; ++qb) first[qb] = cv_fix[qb];
+        for (int qb = 0; qb < C::B_LPW; ++qb) { first[qb] = cv_fix[qb]; first_o[qb] = cv_o[qb]; }
       }
+      conv_tab_write();                       // slab 1 -> table 1
+      __syncthreads();
+      conv_tab_read();
       if (KT > 1) {
 #pragma unroll
         for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(1));
         dma_advance();
       }
       TNX_WAIT_VM(0);
-      if (KT > 0) conv_fixup_all(first, dst0);
-      if (KT > 1) conv_fixup_all(cv_fix, stage_of(1));
+      if (KT > 0) conv_fixup_all(first, first_o, dst0);
+      if (KT > 1) conv_fixup_all(cv_fix, cv_o, stage_of(1));
       cv_pending = false;
+      conv_tab_write();                       // slab 2 -> table 0 (its readers passed the barrier above)
+      __syncthreads();
+      conv_tab_read();
       if (KT > 2) {
 #pragma unroll
         for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(2));
         dma_advance();
       }
+      conv_tab_write();                       // slab 3 -> table 1
       __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the fix-up writes are done before the barrier that follows
       return;
     }

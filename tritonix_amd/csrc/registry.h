@@ -65,12 +65,12 @@ template <class T, class C> struct BtLaunch<T, C, true> {
   static constexpr launch_fn fn = &launch_tile<T, C, true, false, true>;
 };
 
-// The conv2d variant exists for the three-slot 16-bit tiles 128x128, 256x128 and 128x256 with a 128-byte K slab, four
-// or eight waves (256x256 has no registers left for the loader's pixel and filter-tap state with four waves -- it
-// spills inside the K loop -- and three slots of it do not fit the LDS; a 64-channel tile was measured and loses to the
+// The conv2d variant exists for the three-slot, eight-wave 16-bit tiles 128x128, 256x128 and 128x256 with a 128-byte K
+// slab (with four waves it was measured 15-20 % slower, and 256x256 then has no registers left for the loader's state;
+// three slots of 256x256 do not fit the LDS; a 64-channel tile was measured and loses to the
 // register-staged kernel).  The second half of a period must have room for the slotted fix-up of all B ops.
 template <class C> constexpr bool conv_ok() {
-  return C::ES == 2 && (C::NW == 4 || C::NW == 8) && C::KSTEPS * C::TM * C::TN >= 16 &&
+  return C::ES == 2 && C::NW == 8 && C::KSTEPS * C::TM * C::TN >= 16 &&
          C::KSTEPS * C::TM * C::TN / 2 > C::B_LPW + (C::KSTEPS * C::TM * C::TN >= 32 ? 6 : 3) + 1 && C::STAGES == 3 && C::BK == 64 &&
          C::BM >= 128 && C::BN >= 128 && C::TM * C::TN * C::ACC_N <= 128;
 }
