@@ -13,11 +13,11 @@ using namespace tnx;
 extern "C" const ConvGroup* tnx_conv_groups(int* ngroups);      // generated
 extern "C" const KernelGroup* tnx_kernel_groups(int* ngroups);  // generated
 
-// The GEMM kernel's conv2d variant for this tile (three ring slots), or null.  Built with four and with eight waves;
-// eight are taken when built: the loader's address arithmetic and the fix-up are vector instructions in the MFMA
-// stream, and with two waves per SIMD one wave's arithmetic runs under the other's MFMAs (measured on 3x3 layers,
-// batch 32: 256x128 524 -> 620 TFLOP/s at 56x56 / 256 channels, 128x128 248 -> 292 at 28x28 / 128 and 351 -> 420 at
-// 14x14 / 512).
+// The GEMM kernel's conv2d variant for this tile (three ring slots), or null.  Eight waves are preferred (and the
+// only ones built): the loader's address arithmetic and the fix-up are vector instructions in the MFMA stream, and
+// with two waves per SIMD one wave's arithmetic runs under the other's MFMAs (measured on 3x3 layers, batch 32,
+// against four-wave builds: 256x128 524 -> 620 TFLOP/s at 56x56 / 256 channels, 128x128 248 -> 292 at 28x28 / 128
+// and 351 -> 420 at 14x14 / 512).
 static const KernelEntry* find_dma(int dtype, int bcout, int bpix, int bk) {
   int ng = 0;
   const KernelGroup* g = tnx_kernel_groups(&ng);
