@@ -71,6 +71,10 @@ DMA_CASES = {
     "no_pad": (1, 192, 10, 10, 256, 3, 3, (1, 1), (0, 0), (1, 1), True),
     "5x5": (2, 64, 12, 12, 128, 5, 5, (1, 1), (2, 2), (1, 1), False),
     "w_out_3": (2, 64, 3, 3, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    # 1x1, unit strides, no padding: the plane is handed to the kernel as one row (49 and 196 are not multiples of 8:
+    # the last chunk of the tensor crosses its end)
+    "1x1_plane_7x7": (3, 64, 7, 7, 130, 1, 1, (1, 1), (0, 0), (1, 1), True),
+    "1x1_plane_14x14_dilated": (2, 128, 14, 14, 192, 1, 1, (1, 1), (0, 0), (2, 3), False),
 }
 DMA_TILES = [(128, 128, 64), (128, 256, 64), (256, 128, 64)]     # BLOCK_SIZE_M (pixels), BLOCK_SIZE_N (channels), BLOCK_SIZE_K
 

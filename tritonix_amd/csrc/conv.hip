@@ -67,12 +67,34 @@ static void builtin_tile(const tnx_conv2d_args* a, int64_t pixels, int* bcout, i
   *bk = gemm_k > 32 ? 64 : 32;
 }
 
+// The image the direct-to-LDS kernel is given.  A 1x1 filter with unit strides and no padding reads whole planes
+// in order, so the plane is handed over as one row of h*w pixels: the pixel index space then pads h*w, not every
+// row, to a multiple of 8 (14x14: 200 columns per image instead of 224).  Only while h*w fits the kernel's 16-bit
+// pixel coordinates.
+struct DmaImage {
+  int h_in, w_in, h_out, w_out, wp;
+};
+static DmaImage dma_image(const tnx_conv2d_args* a, int h_out, int w_out) {
+  DmaImage g = {a->h_in, a->w_in, h_out, w_out, 0};
+  if (a->filter_h == 1 && a->filter_w == 1 && a->stride_h == 1 && a->stride_w == 1 && a->pad_h == 0 && a->pad_w == 0 &&
+      (int64_t)a->h_in * a->w_in <= 16384) {
+    g.h_in = g.h_out = 1;
+    g.w_in = g.w_out = a->h_in * a->w_in;
+  }
+  g.wp = (g.w_out + 7) / 8 * 8;
+  return g;
+}
+static int64_t dma_cols(const tnx_conv2d_args* a, int h_out, int w_out) {
+  const DmaImage g = dma_image(a, h_out, w_out);
+  return (int64_t)a->batch * g.h_out * g.wp;
+}
+
 // Direct-to-LDS kernel: 256 channels x 128 pixels when that still leaves every CU two tiles, else 128 x 128.
 // Measured on 3x3 layers (batch 32, eight-wave builds): 256x128 620 against 476 TFLOP/s for 128x128 at 56x56 / 256
 // channels, 128x128 ahead of it at 28x28 / 128 channels (292 : 228) and 14x14 / 512 channels (420 : 337), and both
 // well ahead of the register-staged kernel (392, 162, 165) down to a few dozen tiles.
 static bool builtin_dma_tile(const tnx_conv2d_args* a, int h_out, int w_out, int* bcout, int* bpix, int* bk) {
-  const int64_t cols = (int64_t)a->batch * h_out * ((w_out + 7) / 8 * 8);
+  const int64_t cols = dma_cols(a, h_out, w_out);
   const int64_t t256 = ((cols + 127) / 128) * (((int64_t)a->c_out + 255) / 256);
   const int64_t t128 = ((cols + 127) / 128) * (((int64_t)a->c_out + 127) / 128);
   *bpix = 128;
@@ -130,9 +152,8 @@ static int check_problem(const tnx_conv2d_args* a, int32_t* h_out, int32_t* w_ou
 // what the direct-to-LDS kernel needs of the problem (not of the tile)
 static bool dma_problem_ok(const tnx_conv2d_args* a, int h_out, int w_out, bool inspect_ptrs) {
   const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
-  const int64_t wp = (w_out + 7) / 8 * 8;
   if (a->stride_w != 1 || gemm_k % 64 != 0) return false;
-  if ((int64_t)a->batch * h_out * wp >= (1ll << 31) - 4096) return false;
+  if (dma_cols(a, h_out, w_out) >= (1ll << 31) - 4096) return false;
   if (inspect_ptrs && ((uintptr_t)a->weight & 15)) return false;
   // per-lane DMA offsets of the weight slab are 32-bit
   if (256 * gemm_k * 2 >= (1ll << 32)) return false;
@@ -171,7 +192,7 @@ static int resolve(const tnx_conv2d_args* a, Resolved* r, bool inspect_ptrs) {
     want_dma = false;
   }
   if (!want_dma && !reg) return TNX_E_UNSUPPORTED;
-  const int64_t cols = want_dma ? (int64_t)a->batch * h_out * ((w_out + 7) / 8 * 8) : pixels;
+  const int64_t cols = want_dma ? dma_cols(a, h_out, w_out) : pixels;
   if (((cols + bpix - 1) / bpix) * (((int64_t)a->c_out + bcout - 1) / bcout) >= (1ll << 31)) return TNX_E_UNSUPPORTED;
   r->reg = want_dma ? nullptr : reg;
   r->dma = want_dma ? dma : nullptr;
@@ -218,8 +239,8 @@ static void fill_registers(const tnx_conv2d_args* a, const Resolved& r, ConvPara
 
 // GemmParams of the GEMM kernel's conv2d variant: m = c_out, n = padded pixel index, k = c_in * R * S
 static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p, unsigned* grid) {
-  const int h_out = r.h_out, w_out = r.w_out;
-  const int wp = (w_out + 7) / 8 * 8;
+  const DmaImage im = dma_image(a, r.h_out, r.w_out);
+  const int h_out = im.h_out, w_out = im.w_out, wp = im.wp;
   const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
   const int64_t n_total = (int64_t)a->batch * h_out * wp;
   memset(p, 0, sizeof *p);
@@ -235,7 +256,7 @@ static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p,
   p->ktiles_per_split = (int)(gemm_k / r.bk);
   p->out_dtype = a->dtype;
   ConvGeom& g = p->cv;
-  g.h_in = a->h_in; g.w_in = a->w_in; g.c_out = a->c_out; g.h_out = h_out; g.w_out = w_out; g.wp = wp;
+  g.h_in = im.h_in; g.w_in = im.w_in; g.c_out = a->c_out; g.h_out = h_out; g.w_out = w_out; g.wp = wp;
   g.stride_h = a->stride_h; g.pad_h = a->pad_h; g.pad_w = a->pad_w;
   g.hw_in = a->h_in * a->w_in;
   g.chw_in = a->c_in * g.hw_in;
