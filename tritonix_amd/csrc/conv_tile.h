@@ -336,7 +336,7 @@ __global__ __launch_bounds__(C::THREADS, TNX_CONV_OCC) void conv2d_tile_kernel(C
         const int img = (int)fd_div((uint32_t)n, p.div_hw_out);
         const int r0 = n - img * p.hw_out;
         i32x2 v = {(int)(out[0] | ((uint32_t)out[1] << 16)), (int)(out[2] | ((uint32_t)out[3] << 16))};
-        *(i32x2*)(y16 + ((int64_t)img * p.c_out + row) * p.hw_out + r0) = v;
+        __builtin_nontemporal_store(v, (i32x2*)(y16 + ((int64_t)img * p.c_out + row) * p.hw_out + r0));   // written once, never read here
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {

@@ -278,6 +278,19 @@ __device__ __forceinline__ i32x4 load16_agent(__amdgpu_buffer_rsrc_t w, uint32_t
   return __builtin_amdgcn_raw_buffer_load_b128(w, off, 0, CPOL_SC1);
 }
 
+// 16 bytes of C, stored with the non-temporal hint.  C is written once and never read by the kernel; without the
+// hint its lines are kept in the L2 and the memory-side cache and push out operand panels that the other tiles of the
+// round still need.  Measured on the 8192^3 bf16 problem: 1531 -> 1595 TFLOP/s on data-like operands (power-limited),
+// 1712 -> 2026 on all-zero operands (clock at its maximum: the memory side decides); the gated GEMM 1414 -> 1475,
+// int8 2798 -> 2845 TOP/s.  (The same hint on the B *loads* costs 4-20 %: operands are re-read.)
+// A launch whose output the next launch reads at once (the feed-forward block's up-projection) loses that read's
+// cache hits: the block's down-projection runs ~22 us slower, less than the ~30 us its up-projection gains.
+// (A run-time switch `if (keep) plain store else hinted store` is no way to have both: the compiler sinks the two
+// stores into one and drops the hint, measured as the full loss of the gain.)
+typedef i32x4 __attribute__((aligned(2))) i32x4_loose;
+__device__ __forceinline__ void store16_stream(void* dst, i32x4 v) { __builtin_nontemporal_store(v, (i32x4*)dst); }
+__device__ __forceinline__ void store16_stream_loose(void* dst, i32x4 v) { __builtin_nontemporal_store(v, (i32x4_loose*)dst); }
+
 template <int ES> __device__ __forceinline__ i32x2 lds_read_tr(uint32_t addr);
 template <> __device__ __forceinline__ i32x2 lds_read_tr<2>(uint32_t addr) {
   return __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(TNX_LDS(i16x4, addr)));
@@ -564,7 +577,7 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
         if (vec_ok && gc + PK::OUTV <= ncols) {
           i32x4 v;
           __builtin_memcpy(&v, out, 16);
-          *(i32x4*)dst = v;
+          store16_stream(dst, v);
         } else {
 #pragma unroll 1
           for (int x = 0; x < PK::OUTV; ++x)
@@ -651,12 +664,12 @@ __device__ __forceinline__ void epilogue_store_pairs(ACC (&acc)[C::TM][C::TN], u
         if (FULL) {
           i32x4 v;
           __builtin_memcpy(&v, out, 16);
-          *(i32x4*)dst = v;
+          store16_stream(dst, v);
         } else if (gm < m) {
           if (vec_ok && gc + PK::OUTV <= ncols) {
             i32x4 v;
             __builtin_memcpy(&v, out, 16);
-            *(i32x4*)dst = v;
+            store16_stream(dst, v);
           } else {
 #pragma unroll 1
             for (int x = 0; x < PK::OUTV; ++x)
@@ -814,9 +827,9 @@ __device__ __forceinline__ void epilogue_store_conv(ACC (&acc)[C::TM][C::TN], ui
         for (int x = 0; x < 8; ++x) out[x] = O::cvt(f[u][x] + bv);
         raw* dst = yp + (((int64_t)img * g.c_out + gm) * g.h_out + ho) * g.w_out + wq;
         if (valid >= 8) {
-          Loose16 v;
+          i32x4 v;
           __builtin_memcpy(&v, out, 16);
-          *(Loose16*)dst = v;
+          store16_stream_loose(dst, v);    // 2-byte aligned: w_out need not be a multiple of 8
         } else {
 #pragma unroll 1
           for (int x = 0; x < valid; ++x) dst[x] = out[x];
