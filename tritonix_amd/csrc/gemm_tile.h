@@ -886,6 +886,21 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Phase trace (builds with -DTNX_PHASE_TRACE only; tritonix_amd/phase_trace.py reads it): wave 0 of every
+  // workgroup of the one-tile-per-workgroup kernel leaves the 100 MHz timestamp of its start, of the first slab's
+  // arrival, of its last MFMA and of its last store instruction, and the two hardware-id registers that name its
+  // CU, in 64 bytes of the workspace (uncut launches that are handed a workspace only).  (The branch is on the wave id, not the thread id: a divergent branch here
+  // made the compiler carry the DMA base pointers in vector registers, which the loads cannot take.)
+#ifdef TNX_PHASE_TRACE
+#define TNX_PHASE(i) do { if (wave == 0 && p.ws && p.split_k == 1) ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+  if (wave == 0 && p.ws && p.split_k == 1) {
+    ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + 4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID
+    ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);   // XCC_ID
+  }
+  TNX_PHASE(0);
+#else
+#define TNX_PHASE(i)
+#endif
 
   // ---- which tile / split ------------------------------------------------
   // Tiles [0, split_tile0) in launch order are computed whole by one workgroup each; the
@@ -1560,7 +1575,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       issue_prologue();
       if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
     }
+    TNX_PHASE(1);
     k_loop();
+    TNX_PHASE(2);
 
     // ---- epilogue ------------------------------------------------------------
     // every wave is done with the slabs before the LDS is reused for the output strips
@@ -1595,6 +1612,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
                                              p.c_vec_ok, p.epilogue);
     }
+    TNX_PHASE(3);
   } else {
     // ---- persistent: this workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... ------------
     // The host launches it only with KT >= STAGES.  While the epilogue of a tile runs, the first
