@@ -185,6 +185,15 @@ const char* tnx_kernel_name(int i);
 int tnx_probe_mfma(int dtype, int mfma_rows, int zero_operands, int workgroups, int iterations, void* scratch,
                    size_t scratch_bytes, void* stream, double* ops_per_launch);
 
+/* Measurement aid with no counterpart in the reference: one wave issues `iterations` x 8 LDS instructions of one
+ * kind, lane l at byte offset lane_offsets[l] (+ u * 4096, u = 0..7) of a 64 KiB LDS array.  lane_offsets is a HOST
+ * array of 64 offsets, each at most 32768 and aligned to the access (16 bytes for the b128 forms, 8 for the
+ * transposing reads).  Run under `rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_INSTS_LDS`: the
+ * conflict cycles per instruction of that address pattern.  `scratch`: 512 bytes of device memory (table and
+ * don't-care output).  Asynchronous on `stream` after a 256-byte host-to-device copy. */
+enum tnx_lds_op { TNX_LDS_READ_B128 = 0, TNX_LDS_WRITE_B128 = 1, TNX_LDS_READ_TR16_B64 = 2, TNX_LDS_READ_TR8_B64 = 3 };
+int tnx_probe_lds(int op, const uint32_t* lane_offsets, int iterations, void* scratch, size_t scratch_bytes, void* stream);
+
 /* ---- conv2d forward (implicit GEMM on the same LDS layout and MFMA fragments) ------------------------------
  * Stands in for conv2d_forward_kernel, tritonix/ops/conv2d/forward.py:19-165: contiguous NCHW input, KCRS
  * weight, NCHW output of the input's type, GEMM_M = batch * h_out * w_out, GEMM_N = c_out, GEMM_K = c_in *

@@ -6,6 +6,10 @@
 // its power limit and lowers the shader clock, so the rate this loop reaches is an upper bound for
 // any GEMM kernel on such operands -- the kernels in gemm_tile.h add LDS, L2 and HBM traffic on top.
 // With all-zero operands the same loop runs at the full clock.
+//
+// Second aid: one wave issuing one kind of LDS instruction on a caller-given table of per-lane addresses, for the
+// bank-conflict counters (which lanes an instruction serves in one cycle is not documented; the A-slab swizzle in
+// gemm_tile.h is built on what this probe shows).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -16,6 +20,9 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+#define TNX_LDS(T, addr) ((T __attribute__((address_space(3)))*)(uintptr_t)(addr))
 
 __device__ __forceinline__ unsigned mix(unsigned x) {
   x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
@@ -107,7 +114,54 @@ template <int DT> hipError_t launch(int shape, float* out, unsigned grid, int it
   return hipGetLastError();
 }
 
+// One wave, one LDS instruction kind, per-lane byte addresses from a table: eight instructions per iteration at
+// table[lane] + u * 4096 (the multiple of the bank period keeps the pattern).  Read under
+// `rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_INSTS_LDS`: conflict cycles per instruction.
+template <int OP> __global__ __launch_bounds__(64) void lds_pattern_kernel(const uint32_t* table, int iters, int* out) {
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[65536];
+  const uint32_t base = (uint32_t)(uintptr_t)(uint8_t __attribute__((address_space(3)))*)smem;
+  for (int i = threadIdx.x; i < 16384; i += 64) ((int*)smem)[i] = i;
+  __syncthreads();
+  const uint32_t a = base + table[threadIdx.x];
+  i32x4 acc = {0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t addr = a + u * 4096;
+      if (OP == TNX_LDS_READ_B128) acc ^= *TNX_LDS(i32x4, addr);
+      if (OP == TNX_LDS_WRITE_B128) *TNX_LDS(i32x4, addr) = i32x4{it, u, it, u};
+      if (OP == TNX_LDS_READ_TR16_B64) {
+        const i32x2 v = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(TNX_LDS(i16x4, addr)));
+        acc.x ^= v.x, acc.y ^= v.y;
+      }
+      if (OP == TNX_LDS_READ_TR8_B64) {
+        const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(TNX_LDS(i32x2, addr));
+        acc.x ^= v.x, acc.y ^= v.y;
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+  out[threadIdx.x] = acc.x ^ acc.y ^ acc.z ^ acc.w;
+}
+
 }  // namespace
+
+extern "C" int tnx_probe_lds(int op, const uint32_t* lane_offsets, int iterations, void* scratch, size_t scratch_bytes,
+                             void* stream) {
+  if (op < TNX_LDS_READ_B128 || op > TNX_LDS_READ_TR8_B64 || !lane_offsets || iterations <= 0 || !scratch) return TNX_E_INVALID;
+  if (scratch_bytes < 512) return TNX_E_WORKSPACE;
+  for (int l = 0; l < 64; ++l)
+    if (lane_offsets[l] > 32768u || (lane_offsets[l] & (op <= TNX_LDS_WRITE_B128 ? 15u : 7u))) return TNX_E_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t* table = (uint32_t*)scratch;
+  int* out = (int*)scratch + 64;
+  if (hipMemcpyAsync(table, lane_offsets, 256, hipMemcpyHostToDevice, s) != hipSuccess) return TNX_E_HIP;
+  if (op == TNX_LDS_READ_B128) hipLaunchKernelGGL((lds_pattern_kernel<TNX_LDS_READ_B128>), dim3(1), dim3(64), 0, s, table, iterations, out);
+  else if (op == TNX_LDS_WRITE_B128) hipLaunchKernelGGL((lds_pattern_kernel<TNX_LDS_WRITE_B128>), dim3(1), dim3(64), 0, s, table, iterations, out);
+  else if (op == TNX_LDS_READ_TR16_B64) hipLaunchKernelGGL((lds_pattern_kernel<TNX_LDS_READ_TR16_B64>), dim3(1), dim3(64), 0, s, table, iterations, out);
+  else hipLaunchKernelGGL((lds_pattern_kernel<TNX_LDS_READ_TR8_B64>), dim3(1), dim3(64), 0, s, table, iterations, out);
+  return hipGetLastError() == hipSuccess ? TNX_OK : TNX_E_HIP;
+}
 
 extern "C" int tnx_probe_mfma(int dtype, int mfma_rows, int zero_operands, int workgroups, int iterations, void* scratch,
                               size_t scratch_bytes, void* stream, double* ops_per_launch) {
