@@ -245,3 +245,23 @@ def test_unforced_dispatch_never_selects_the_vendor_library(device, name, scale,
     else:
         assert oracle.within_tolerance(out, ref)[0]
     matmul.clear_cache()
+
+
+@pytest.mark.gpu
+def test_measurement_probes_launch_and_finish(device):
+    """tnx_probe_mfma and tnx_probe_lds are launched by bench.py and the LDS probe script: both must run to completion."""
+    import ctypes
+
+    from tritonix_amd import _C, lds_probe
+
+    lib = _C.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    scratch = torch.zeros(8 * 256, dtype=torch.float32, device=device)
+    ops = ctypes.c_double(0)
+    assert lib.tnx_probe_mfma(_C.BF16, 16, 0, 8, 4, scratch.data_ptr(), scratch.numel() * 4, stream, ctypes.byref(ops)) == _C.OK
+    assert ops.value == 8 * 4 * 4 * 2.0 * 128 * 128 * 32
+    for name, op, offs in lds_probe.patterns()[:10]:
+        table = (ctypes.c_uint32 * 64)(*offs)
+        assert lib.tnx_probe_lds(op, table, 4, scratch.data_ptr(), 512, stream) == _C.OK, name
+        torch.cuda.synchronize()
+        assert scratch[:64].view(torch.int32).tolist() == offs      # the table the kernel read
