@@ -118,7 +118,19 @@ typedef struct tnx_gemm_args {
  * CU count (the reference's answer to the same problem is a persistent kernel,
  * playground/persistent_mma.py:47-141). */
 
-/* Launch one GEMM.  Returns a tnx_status.  Asynchronous. */
+/* Launch one GEMM.  Returns a tnx_status.  Asynchronous.
+ * Which loader moves the operands follows from their layout, not from an argument:
+ *   - A row-major (stride_ak == 1) and B row-major (stride_bn == 1): the direct-to-LDS loader of every built tile.
+ *     With K a multiple of block_k, 16-byte aligned rows and base pointers and N a multiple of 16 bytes of elements
+ *     every K slab goes through it; otherwise (16-bit types: any 2-byte-aligned rows and pointers, any K and N;
+ *     int8: rows and pointers still 16-byte aligned, any K and N; row pitches at least the row length) the last K
+ *     slab is loaded element by element with zero fill and the slabs before it through the direct loader.
+ *     TNX_SCHED_PERSISTENT takes the first form only.
+ *   - A row-major and B k-contiguous (stride_bk == 1, the view w.t() of a row-major weight) with K a multiple of
+ *     block_k and 16-byte aligned rows and pointers: a direct-to-LDS loader of its own, in the tiles whose K slab is
+ *     128 bytes per row.
+ *   - anything else (strided A, overlapping rows, ...): the element-wise loader, built for two tiles per type
+ *     (128x128 and 64x128, four waves, two stages); other tiles return TNX_E_UNSUPPORTED. */
 int tnx_gemm(const tnx_gemm_args* args);
 
 /* tnx_gemm without any allocation on anyone's side.  No counterpart in the reference: it is for callers

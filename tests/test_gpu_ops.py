@@ -215,16 +215,20 @@ def test_memoised_config_follows_the_operand_layout(device, monkeypatch):
     assert torch.equal(out1, out3)
     # row-major B (class 1) and k-contiguous B (class 2) are remembered apart
     assert (512, 384, 256, torch.float16, 1) in mm._matmul_cfg and (512, 384, 256, torch.float16, 2) in mm._matmul_cfg
-    # a misaligned base pointer is the second layout class too
+    # a misaligned base pointer is a class of its own: the DMA loader with an element-wise last K slab
     flat = torch.zeros(512 * 256 + 8, dtype=torch.float16, device=device)
     a_off = flat[1:1 + 512 * 256].view(512, 256)
     a_off.copy_(ad)
-    assert mm.dma_layout(a_off, b_contig) == 0 and mm.dma_layout(ad, b_contig) == 1 and mm.dma_layout(ad, wd.t()) == 2
-    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_off, b_contig), ref)[0]
+    assert mm.dma_layout(a_off, b_contig) == 3 and mm.dma_layout(ad, b_contig) == 1 and mm.dma_layout(ad, wd.t()) == 2
+    assert torch.equal(tritonix_amd.triton_matmul(a_off, b_contig), out1)
+    # a column-major A is none of the DMA layouts: the two tiles built with the element-wise loader
+    a_cm = ad.t().contiguous().t()
+    assert a_cm.stride() == (1, 512) and mm.dma_layout(a_cm, b_contig) == 0
+    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_cm, b_contig), ref)[0]
     # a memo entry the engine refuses for these operands is replaced, not raised
     mm._matmul_cfg[(512, 384, 256, torch.float16, 0)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, 1)],
                                                              block_m=256, block_n=256, num_stages=2, num_warps=4)
-    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_off, b_contig), ref)[0]
+    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_cm, b_contig), ref)[0]
     assert mm._matmul_cfg[(512, 384, 256, torch.float16, 0)]["block_m"] == 128       # replaced by the built-in choice
     mm._matmul_cfg.clear()
 

@@ -247,11 +247,63 @@ def test_error_mapping_on_launch(device):
     with pytest.raises(ValueError):
         gemm(a, a, cfg(96, 128, 64, 4, 2))            # no such tile
     with pytest.raises(ValueError):
-        gemm(a[:, :200], a[:200], cfg(128, 128, 64, 4, 3))   # ragged K on a DMA-only tile
+        gemm(a[:, :200].t(), a[:200], cfg(128, 128, 64, 4, 3))   # strided A on a DMA-only tile
     with pytest.raises(ValueError):
         gemm(a.float(), a.float(), GENERIC)
     with pytest.raises(ValueError):
         gemm(a.cpu(), a.cpu(), GENERIC)
+
+
+# ---- row-major operands the DMA loader takes with an element-wise last K slab ---------------
+@pytest.mark.parametrize("dtype,tile,shape,off,pad,split", [
+    (torch.bfloat16, (256, 256, 64, 4, 2), (1000, 1100, 1032), (0, 0), (0, 0), 1),      # K = 16 slabs + 8
+    (torch.bfloat16, (256, 256, 64, 8, 2), (520, 1304, 1028), (0, 0), (0, 0), 1),       # rows of A 8 bytes off
+    (torch.bfloat16, (256, 128, 64, 4, 3), (512, 1030, 1024), (0, 0), (0, 0), 1),       # N ends inside a chunk, K whole
+    (torch.bfloat16, (128, 128, 64, 4, 3), (700, 517, 1031), (5, 7), (3, 5), 1),        # everything odd, views into larger buffers
+    (torch.float16, (64, 64, 64, 4, 4), (300, 200, 40), (1, 1), (0, 0), 1),             # K shorter than one slab
+    (torch.bfloat16, (128, 128, 64, 4, 3), (512, 1024, 4135), (0, 0), (0, 0), 8),       # K cut eight ways, the tail in the last slice
+    (torch.bfloat16, (64, 128, 64, 8, 3), (16, 4096, 14340), (0, 0), (0, 0), 8),        # the skinny benchmark shape plus four
+    (torch.int8, (256, 256, 128, 4, 2), (600, 1000, 1168), (0, 0), (0, 8), 1),          # int8: ragged K and N, rows 16-byte aligned
+    (torch.int8, (64, 128, 128, 4, 3), (64, 2051, 2064), (0, 0), (0, 13), 1),
+], ids=lambda v: str(v).replace("torch.", "").replace(" ", ""))
+def test_ragged_row_major_operands_on_the_dma_path(device, dtype, tile, shape, off, pad, split):
+    """What surrounds the operands in memory is NaN (int8: 77): nothing of it may reach C.  A second launch on
+    zero-padded, aligned copies runs the ordinary DMA path; slab by slab both add the same products in the same
+    order, so the two results have to agree bit for bit."""
+    m, n, k = shape
+    g = torch.Generator("cpu").manual_seed(m + 3 * n + 7 * k)
+    fill = 77 if dtype == torch.int8 else float("nan")
+    if dtype == torch.int8:
+        a = torch.randint(-127, 128, (m, k), generator=g, dtype=dtype)
+        b = torch.randint(-127, 128, (k, n), generator=g, dtype=dtype)
+    else:
+        a = torch.randn(m, k, generator=g).to(dtype)
+        b = (torch.randn(k, n, generator=g) / k ** 0.5).to(dtype)
+    abuf = torch.full((m * (k + pad[0]) + 64,), fill, dtype=dtype)
+    bbuf = torch.full((k * (n + pad[1]) + 64,), fill, dtype=dtype)
+    av = abuf[off[0]:off[0] + m * (k + pad[0])].view(m, k + pad[0])
+    bv = bbuf[off[1]:off[1] + k * (n + pad[1])].view(k, n + pad[1])
+    av[:, :k] = a
+    bv[:, :n] = b
+    ad = abuf.to(device)[off[0]:off[0] + m * (k + pad[0])].view(m, k + pad[0])[:, :k]
+    bd = bbuf.to(device)[off[1]:off[1] + k * (n + pad[1])].view(k, n + pad[1])[:, :n]
+    extra = dict(split_k=split) if split > 1 else {}
+    kernel = gemm_splitk_kernel if split > 1 else matmul_kernel
+    out = gemm(ad, bd, cfg(*tile, **extra), kernel=kernel)
+    ref = oracle.reference_matmul(a, b)
+    if dtype == torch.int8:
+        assert torch.equal(out.cpu(), ref)
+    else:
+        assert bool(torch.isfinite(out.float()).all())
+        check_fp(out, ref)
+    bk = tile[2]
+    kp, npad = -(-k // bk) * bk, -(-n // 16) * 16
+    ap = torch.zeros((m, kp), dtype=dtype)
+    bp = torch.zeros((kp, npad), dtype=dtype)
+    ap[:, :k] = a
+    bp[:k, :n] = b
+    want = gemm(ap.to(device), bp.to(device), cfg(*tile, **extra), kernel=kernel)[:, :n]
+    assert torch.equal(out, want)
 
 
 # ---- K cut only for the trailing tiles (fills the last, partial wave of workgroups) ------

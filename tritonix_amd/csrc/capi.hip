@@ -79,21 +79,32 @@ static int check_common(const tnx_gemm_args* a) {
 // Which DMA loader the operands can take: 0 = none (element-wise loader only), 1 = row-major B
 // (stride_bn == 1), 2 = k-contiguous B (stride_bk == 1, the layout of x @ w.t()).  Both need row-major A,
 // 16-byte aligned rows and base pointers and k % block_k == 0.
-static int dma_layout(const tnx_gemm_args* a) {
+// 0: element-wise loader; 1: DMA loader, A and B row-major; 2: DMA loader, B k-contiguous.
+// *tail (layout 1 only): the operands are row-major but not as the DMA loader likes them best -- K no multiple of
+// block_k, rows or base pointers of 16-bit operands not 16-byte aligned (the loads take any 2-byte-aligned address),
+// N ending inside a 16-byte chunk -- so the last K slab, the only one whose chunks can cross the end of a row of A
+// or of the last row of B, is loaded element by element instead (GemmParams::tail_slab).
+static int dma_layout(const tnx_gemm_args* a, bool* tail = nullptr) {
   const int es = elem_size(a->in_dtype);
   const int vec = 16 / es;
-  if (a->stride_ak != 1) return 0;
-  if (a->k % a->block_k != 0 || a->k == 0) return 0;
-  if ((a->stride_am * es) % 16 != 0 || a->stride_am < 0) return 0;
-  if (((uintptr_t)a->a & 15) || ((uintptr_t)a->b & 15)) return 0;
+  if (tail) *tail = false;
+  if (a->stride_ak != 1 || a->k == 0 || a->stride_am < 0) return 0;
   // per-lane DMA offsets are 32-bit
   if ((int64_t)a->block_m * a->stride_am * es >= (1ll << 32)) return 0;
-  if (a->stride_bn == 1) {
-    if ((a->stride_bk * es) % 16 != 0 || a->stride_bk < 0) return 0;
-    if (a->n % vec != 0 || a->n < vec) return 0;
-    if ((int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es >= (1ll << 32)) return 0;
-    return 1;
+  const bool a_aligned = (a->stride_am * es) % 16 == 0 && !((uintptr_t)a->a & 15) && !((uintptr_t)a->b & 15);
+  if (a->stride_bn == 1 && a->stride_bk >= 0 &&
+      (int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es < (1ll << 32)) {
+    const bool strict = a_aligned && a->k % a->block_k == 0 && (a->stride_bk * es) % 16 == 0 && a->n % vec == 0 && a->n >= vec;
+    if (strict) return 1;
+    // int8 operands keep 16-byte aligned rows (1-byte-aligned DMA addresses are untried); only K and N may be ragged
+    const bool loose_ok = tail && (es == 2 || (a_aligned && (a->stride_bk * es) % 16 == 0)) && a->stride_am >= a->k &&
+                          a->stride_bk >= a->n;
+    if (loose_ok) {
+      *tail = true;
+      return 1;
+    }
   }
+  if (a->k % a->block_k != 0 || !a_aligned) return 0;
   if (a->stride_bk == 1) {
     if ((a->stride_bn * es) % 16 != 0 || a->stride_bn < 0) return 0;
     if ((int64_t)a->block_n * a->stride_bn * es + (int64_t)a->block_k * es >= (1ll << 32)) return 0;
@@ -121,8 +132,10 @@ extern "C" size_t tnx_gemm_workspace_bytes(const tnx_gemm_args* a) {
   return (size_t)WS_COUNTER_BYTES + (size_t)a->split_k * (size_t)cut_tiles(a) * (size_t)a->block_m * (size_t)a->block_n * 4;
 }
 
-static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs, bool* bt = nullptr) {
+static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool* fast, bool inspect_ptrs, bool* bt = nullptr,
+                          bool* tail = nullptr) {
   if (bt) *bt = false;
+  if (tail) *tail = false;
   int st = check_common(a);
   if (st != TNX_OK) return st;
   int64_t lds = lds_bytes_of(a);
@@ -147,7 +160,10 @@ static int supported_impl(const tnx_gemm_args* a, const KernelEntry** out, bool*
   if (!e) return TNX_E_UNSUPPORTED;
   tnx_gemm_args tmp = *a;
   if (!inspect_ptrs) { tmp.a = nullptr; tmp.b = nullptr; }
-  const int layout = dma_layout(&tmp);
+  bool tail_slab = false;
+  // the persistent kernel keeps the strict layout
+  const int layout = dma_layout(&tmp, (a->schedule & TNX_SCHED_PERSISTENT) ? nullptr : &tail_slab);
+  if (tail) *tail = tail_slab;
   bool f = layout == 1 || (layout == 2 && e->fast_bt);
   if (!f && !e->generic) return TNX_E_UNSUPPORTED;
   if (a->schedule & TNX_SCHED_PERSISTENT) {
@@ -184,8 +200,8 @@ extern "C" int tnx_gemm_supported(const tnx_gemm_args* a) { return supported_imp
 
 extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   const KernelEntry* e = nullptr;
-  bool fast = false, bt = false;
-  int st = supported_impl(a, &e, &fast, true, &bt);
+  bool fast = false, bt = false, tail_slab = false;
+  int st = supported_impl(a, &e, &fast, true, &bt, &tail_slab);
   if (st != TNX_OK) return st;
   if (!a->a || !a->b || !a->c) {
     if (a->m == 0 || a->n == 0) return TNX_OK;
@@ -221,6 +237,8 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.tile_order = (a->schedule & TNX_SCHED_SUPERBLOCK) && a->split_k == 1 ? 1 : 0;
   p.atomic_reduce = (a->schedule & TNX_SCHED_ATOMIC_REDUCE) && a->split_k > 1 ? 1 : 0;
   p.c_vec_ok = a->stride_cn == 1 && ((a->stride_cm * es_out) % 16) == 0 && (((uintptr_t)a->c) % 16) == 0;
+  p.c_row_ok = a->stride_cn == 1;
+  p.tail_slab = tail_slab ? 1 : 0;
 
   hipStream_t stream = (hipStream_t)a->stream;
   hipError_t err;
@@ -316,7 +334,8 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     tnx_gemm_args t = *a;   // a and b, when given, count with their base alignment (null = aligned)
     if (t.stride_ak == 0 && t.stride_bn == 0) { t.stride_am = t.k; t.stride_ak = 1; t.stride_bk = t.n; t.stride_bn = 1; }
     t.block_m = 128; t.block_n = 128; t.block_k = bk;
-    dma_ok = dma_layout(&t) != 0;     // every tile the choice below proposes is built for both DMA layouts
+    bool tail_slab = false;
+    dma_ok = dma_layout(&t, &tail_slab) != 0;     // every tile the choice below proposes is built for both DMA layouts
   }
   if (a->m <= 64 && dma_ok) {
     // skinny: B is streamed once; K is split until every CU owns one workgroup (measured on the
@@ -329,8 +348,8 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     a->split_k = s;
     return TNX_OK;
   }
-  // operands the DMA loader cannot take (ragged K, odd strides or widths) go to one of the two
-  // tiles that are also built with the element-wise loader
+  // operands the DMA loader cannot take (not row-major with unit inner strides, int8 rows that are not 16-byte
+  // aligned) go to one of the two tiles that are also built with the element-wise loader
   if (!dma_ok) {
     a->block_m = a->m <= 64 ? 64 : 128; a->block_n = 128; a->num_stages = 2; a->num_warps = 4;
     return TNX_OK;

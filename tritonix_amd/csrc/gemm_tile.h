@@ -18,6 +18,7 @@
 //     group-M order of tl.swizzle2d (tritonix/ops/matmul.py:70).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 namespace tnx {
@@ -94,6 +95,8 @@ struct GemmParams {
   int epilogue;
   int out_dtype;
   bool c_vec_ok;          // C takes 16-byte stores along n (stride_cn == 1, 16-byte aligned rows)
+  bool c_row_ok;          // stride_cn == 1: rows of C take 16-byte stores at the element's own alignment
+  int tail_slab;          // DMA kernels: the last K slab (whole or partial) goes through the element-wise loader
   bool b_once;            // every element of B is read by exactly one workgroup (one tile row): stream it non-temporally
   int tile_order;         // 0: XCD remap + tl.swizzle2d(group_m); 1: 16x16 super-blocks in serpentine order (superblock_order)
   int atomic_reduce;      // split-K: slices are added into one fp32/int32 copy with device-scope atomics instead of being kept apart
@@ -288,6 +291,7 @@ __device__ __forceinline__ i32x4 load16_agent(__amdgpu_buffer_rsrc_t w, uint32_t
 // (A run-time switch `if (keep) plain store else hinted store` is no way to have both: the compiler sinks the two
 // stores into one and drops the hint, measured as the full loss of the gain.)
 typedef i32x4 __attribute__((aligned(2))) i32x4_loose;
+typedef i32x4 __attribute__((aligned(1))) i32x4_bytes;
 __device__ __forceinline__ void store16_stream(void* dst, i32x4 v) { __builtin_nontemporal_store(v, (i32x4*)dst); }
 __device__ __forceinline__ void store16_stream_loose(void* dst, i32x4 v) { __builtin_nontemporal_store(v, (i32x4_loose*)dst); }
 
@@ -584,7 +588,7 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
         if (vec_ok && gc + PK::OUTV <= ncols) {
           i32x4 v;
           __builtin_memcpy(&v, out, 16);
-          store16_stream(dst, v);
+          store16_stream_loose(dst, v);                 // rows of C need not be 16-byte aligned
         } else {
 #pragma unroll 1
           for (int x = 0; x < PK::OUTV; ++x)
@@ -947,10 +951,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int kt0 = cut ? split * p.ktiles_per_split : 0;
   int kt1 = cut ? kt0 + p.ktiles_per_split : kt_total;
   if (kt1 > kt_total) kt1 = kt_total;
-  const int KT = kt1 > kt0 ? kt1 - kt0 : 0;          // slabs of this workgroup (per tile)
-  // FAST kernels are only launched when k % BK == 0 and A, B are row-major
-  // and 16-byte aligned: every slab goes through the DMA path.  Otherwise every
-  // slab goes through the element-wise loader.
+  // FAST kernels move their slabs with the DMA loader.  It wants chunks that lie inside their row: with a K that is
+  // no multiple of BK, rows that are not 16-byte aligned or an N that ends inside a chunk, the host sets tail_slab
+  // and the last slab of the K range (the only one whose chunks can cross the end of a row of A, or the end of the
+  // last row of B) is left out of the ring and loaded element by element, zero-filled, after the K loop.
+  const bool tail_here = FAST && !PERSIST && !BT && !CONV && p.tail_slab != 0 && kt1 == kt_total && kt1 > kt0;
+  const int KT = kt1 > kt0 ? kt1 - kt0 - (tail_here ? 1 : 0) : 0;          // slabs of this workgroup in the ring (per tile)
 
   // ---- the tile the loader works on: origin, DMA bases and per-lane byte offsets.
   // (In the persistent kernel the loader moves on to the next tile before the epilogue of the
@@ -1055,7 +1061,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         } else {
           int row = P / C::CPR_B, cs = P % C::CPR_B;
           int c = cs ^ C::swzB(row);
-          if (n0 + (int64_t)(c + 1) * (16 / ES) > p.n) c = 0;  // column chunk past N: any valid address
+          // column chunk past N: any valid address.  (A chunk that starts below N and ends above it -- tail_slab
+          // launches only -- is loaded as it is: its upper elements come from the next k row, which exists because
+          // the last slab is not loaded here, and belong to columns that are never stored.)
+          if (n0 + (int64_t)c * (16 / ES) >= p.n || (!p.tail_slab && n0 + (int64_t)(c + 1) * (16 / ES) > p.n)) c = 0;
           b_voff[q] = (uint32_t)((int64_t)row * ldb * ES + c * 16);
         }
       }
@@ -1063,37 +1072,50 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   };
   place_tile(pid_m, pid_n);
 
-  // element-wise loader: any strides, any ragged edge, zero fill.  Used for
-  // the K-tail slab of FAST kernels and for every slab otherwise.
-  auto load_slab_generic = [&](int kt_global, uint32_t stage_base) __attribute__((always_inline)) {
+  // Loader for what the DMA path does not take: any strides, any ragged edge, zero fill.  One 16-byte chunk of the
+  // slab per thread and trip: a chunk that lies inside the matrix along a unit-stride dimension is one vector load
+  // at the element's own alignment, any other chunk is put together element by element.  Used for every slab of the
+  // kernels built without the DMA loader and for the left-out last slab of a tail_slab launch.
+  // (t0: the thread's index in the workgroup, handed in so that the DMA kernels need not keep threadIdx.x alive
+  // across their K loop for the one call after it)
+  auto load_slab_generic = [&](int kt_global, uint32_t stage_base, int t0) __attribute__((always_inline)) {
+    typedef typename std::conditional<ES == 2, uint16_t, uint8_t>::type elem_t;
+    typedef typename std::conditional<ES == 2, i32x4_loose, i32x4_bytes>::type chunk_t;
+    constexpr int EPC = 16 / ES;                         // elements per chunk
     const int64_t k0 = (int64_t)kt_global * BK;
-    for (int idx = tid; idx < BM * BK; idx += C::THREADS) {
-      int row = idx / BK, kk = idx % BK;
-      int64_t gm = m0 + row, gk = k0 + kk;
-      uint32_t dst = stage_base + row * C::ROWB_A + ((((kk * ES) >> 4) ^ C::swzA(row)) << 4) + ((kk * ES) & 15);
-      if (ES == 2) {
-        uint16_t v = 0;
-        if (gm < p.m && gk < p.k) v = ((const uint16_t*)p.a)[gm * p.sam + gk * p.sak];
-        *TNX_LDS(uint16_t, dst) = v;
-      } else {
-        uint8_t v = 0;
-        if (gm < p.m && gk < p.k) v = p.a[gm * p.sam + gk * p.sak];
-        *TNX_LDS(uint8_t, dst) = v;
+    const elem_t* ap = (const elem_t*)p.a;
+    const elem_t* bp = (const elem_t*)p.b;
+    for (int idx = t0; idx < BM * C::CPR_A; idx += C::THREADS) {
+      const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
+      const int64_t gm = m0 + row, gk = k0 + cs * EPC;
+      i32x4 v = {0, 0, 0, 0};
+      if (gm < p.m && gk < p.k) {
+        if (p.sak == 1 && gk + EPC <= p.k) {
+          v = *(const chunk_t*)(ap + gm * p.sam + gk);
+        } else {
+          elem_t e[EPC];
+#pragma unroll
+          for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? ap[gm * p.sam + (gk + x) * p.sak] : (elem_t)0;
+          __builtin_memcpy(&v, e, 16);
+        }
       }
+      *TNX_LDS(i32x4, stage_base + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
     }
-    for (int idx = tid; idx < BK * BN; idx += C::THREADS) {
-      int row = idx / BN, nn = idx % BN;
-      int64_t gk = k0 + row, gn = n0 + nn;
-      uint32_t dst = stage_base + C::A_BYTES + row * C::ROWB_B + ((((nn * ES) >> 4) ^ C::swzB(row)) << 4) + ((nn * ES) & 15);
-      if (ES == 2) {
-        uint16_t v = 0;
-        if (gk < p.k && gn < p.n) v = ((const uint16_t*)p.b)[gk * p.sbk + gn * p.sbn];
-        *TNX_LDS(uint16_t, dst) = v;
-      } else {
-        uint8_t v = 0;
-        if (gk < p.k && gn < p.n) v = p.b[gk * p.sbk + gn * p.sbn];
-        *TNX_LDS(uint8_t, dst) = v;
+    for (int idx = t0; idx < BK * C::CPR_B; idx += C::THREADS) {
+      const int row = idx / C::CPR_B, cs = idx % C::CPR_B;
+      const int64_t gk = k0 + row, gn = n0 + cs * EPC;
+      i32x4 v = {0, 0, 0, 0};
+      if (gk < p.k && gn < p.n) {
+        if (p.sbn == 1 && gn + EPC <= p.n) {
+          v = *(const chunk_t*)(bp + gk * p.sbk + gn);
+        } else {
+          elem_t e[EPC];
+#pragma unroll
+          for (int x = 0; x < EPC; ++x) e[x] = gn + x < p.n ? bp[gk * p.sbk + (gn + x) * p.sbn] : (elem_t)0;
+          __builtin_memcpy(&v, e, 16);
+        }
       }
+      *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_B + ((cs ^ C::swzB(row)) << 4)) = v;
     }
   };
 
@@ -1489,7 +1511,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
           for (int q = 0; q < C::LPW; ++q) dma_op(q, stage_of(s));
           dma_advance();
         } else {
-          load_slab_generic(kt0 + s, stage_of(s));
+          load_slab_generic(kt0 + s, stage_of(s), tid);
         }
       }
     }
@@ -1548,7 +1570,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
     conv_period_begin();
     const uint32_t dst = stage_of(t);
-    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst);
+    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst, tid);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
     if constexpr (FAST) {
       last_step(sa1, sb1, Yes{}, dst, Par0{}, Yes{});
@@ -1584,6 +1606,22 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
     TNX_PHASE(1);
     k_loop();
+    if constexpr (FAST && !BT && !CONV) {
+      if (tail_here) {
+        // the left-out slab: every wave is done with the ring, slot 0 takes it, one slab of MFMAs follows
+        __syncthreads();
+        load_slab_generic(kt1 - 1, stage_of(0), wave * 64 + lane);
+        __syncthreads();
+        const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ++ks) {
+#pragma unroll
+          for (int idx = 0; idx < NREAD; ++idx) read_one(0, idx, sa, sb, ks);
+#pragma unroll
+          for (int x = 0; x < NMMA; ++x) mma_one(0, x);
+        }
+      }
+    }
     TNX_PHASE(2);
 
     // ---- epilogue ------------------------------------------------------------
@@ -1607,17 +1645,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         return;
       const SliceSrc src = {wave0, (uint32_t)slice_stride, atomic ? 1 : p.split_k, atomic};
       if (p.epilogue == EPI_NONE)
-        epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+        epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0);
       else
         epilogue_store<T, C, O, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                            p.c_vec_ok, p.epilogue);
+                                            p.c_row_ok, p.epilogue);
     } else {
       const SliceSrc none = {nullptr, 0, 0, false};
       if (p.epilogue == EPI_NONE)
-        epilogue_store<T, C, O, false, false>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_vec_ok, 0);
+        epilogue_store<T, C, O, false, false>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0);
       else
         epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                             p.c_vec_ok, p.epilogue);
+                                             p.c_row_ok, p.epilogue);
     }
     TNX_PHASE(3);
   } else {
