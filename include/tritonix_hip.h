@@ -126,9 +126,9 @@ typedef struct tnx_gemm_args {
  *     int8: rows and pointers still 16-byte aligned, any K and N; row pitches at least the row length) the last K
  *     slab is loaded element by element with zero fill and the slabs before it through the direct loader.
  *     TNX_SCHED_PERSISTENT takes the first form only.
- *   - A row-major and B k-contiguous (stride_bk == 1, the view w.t() of a row-major weight) with K a multiple of
- *     block_k and 16-byte aligned rows and pointers: a direct-to-LDS loader of its own, in the tiles whose K slab is
- *     128 bytes per row.
+ *   - A row-major and B k-contiguous (stride_bk == 1, the view w.t() of a row-major weight): a direct-to-LDS loader
+ *     of its own, in the tiles whose K slab is 128 bytes per row, under the same two sets of conditions (K a multiple
+ *     of block_k and 16-byte aligned rows and pointers, or else the last K slab loaded chunk by chunk).
  *   - anything else (strided A, overlapping rows, ...): the element-wise loader, built for two tiles per type
  *     (128x128 and 64x128, four waves, two stages); other tiles return TNX_E_UNSUPPORTED. */
 int tnx_gemm(const tnx_gemm_args* args);

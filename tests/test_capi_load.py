@@ -96,12 +96,13 @@ def test_ragged_layouts_need_a_generic_kernel():
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500, **i8))) == _C.E_UNSUPPORTED
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=400, num_stages=3))) == _C.E_UNSUPPORTED   # rows overlap
     # k-contiguous B (w.t() of a row-major weight) has a DMA loader of its own in every tile whose K slab is 128 bytes
-    # per row; with rows that are not 16-byte aligned it needs the element-wise loader again
+    # per row, 16-bit rows at any alignment included
     assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=512))) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=512, num_warps=8))) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=512, block_k=32, num_stages=3))) == _C.E_UNSUPPORTED
-    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=516))) == _C.OK          # 128x128x64 w4 s2 generic
-    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=516, num_warps=8))) == _C.E_UNSUPPORTED
+    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=516))) == _C.OK
+    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=516, num_warps=8))) == _C.OK
+    assert lib.tnx_gemm_supported(ctypes.byref(args(stride_bk=1, stride_bn=500, num_warps=8))) == _C.E_UNSUPPORTED   # rows of w overlap
     # strided A: element-wise loader only
     assert lib.tnx_gemm_supported(ctypes.byref(args(stride_am=1, stride_ak=512, num_warps=8))) == _C.E_UNSUPPORTED
 

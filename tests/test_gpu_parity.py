@@ -374,6 +374,10 @@ def test_skinny_wave_split_kernel(device, m, n, k, stages, dtype):
     (torch.int8, (256, 256, 128, 4, 2), (1024, 1000, 1024)),
     (torch.int8, (64, 128, 128, 4, 3), (64, 2051, 2048)),
     (torch.bfloat16, (64, 128, 64, 8, 3), (16, 4096, 14336)),      # the skinny benchmark shape against w.t(), K cut 8 ways
+    (torch.bfloat16, (256, 256, 64, 4, 2), (1000, 1100, 1032)),    # K = 16 slabs + 8: the last slab is loaded chunk by chunk
+    (torch.bfloat16, (128, 128, 64, 4, 3), (520, 1304, 1031)),     # rows of A and of w two bytes off 16
+    (torch.int8, (256, 256, 128, 4, 2), (600, 1000, 1168)),        # int8: ragged K, rows 16-byte aligned
+    (torch.bfloat16, (64, 128, 64, 8, 3), (16, 4096, 14340)),      # skinny, K cut 8 ways, ragged K
 ], ids=lambda v: str(v).replace("torch.", "").replace(" ", ""))
 def test_k_contiguous_b_takes_its_own_dma_loader(device, dtype, tile, shape):
     m, n, k = shape
@@ -395,6 +399,10 @@ def test_k_contiguous_b_takes_its_own_dma_loader(device, dtype, tile, shape):
         assert torch.equal(out.cpu(), ref)
     else:
         check_fp(out, ref)
+    # the same products in the same order as with a row-major copy of B (int8 rows of that copy have to be 16-byte
+    # aligned for the tiles without the element-wise loader)
+    if dtype != torch.int8 or n % 16 == 0:
+        assert torch.equal(out, gemm(ad, b.contiguous(), cfg(*tile, **extra), kernel=kernel))
         if n % 8 == 0:
             # the same K order as the row-major loader on a contiguous copy: the same bits
             assert torch.equal(out, gemm(ad, b.contiguous(), cfg(*tile, **extra), kernel=kernel))

@@ -104,11 +104,13 @@ static int dma_layout(const tnx_gemm_args* a, bool* tail = nullptr) {
       return 1;
     }
   }
-  if (a->k % a->block_k != 0 || !a_aligned) return 0;
-  if (a->stride_bk == 1) {
-    if ((a->stride_bn * es) % 16 != 0 || a->stride_bn < 0) return 0;
-    if ((int64_t)a->block_n * a->stride_bn * es + (int64_t)a->block_k * es >= (1ll << 32)) return 0;
-    return 2;
+  if (a->stride_bk == 1 && a->stride_bn >= 0 && (int64_t)a->block_n * a->stride_bn * es + (int64_t)a->block_k * es < (1ll << 32)) {
+    if (a_aligned && a->k % a->block_k == 0 && (a->stride_bn * es) % 16 == 0) return 2;
+    // the same relaxation for a k-contiguous B: rows of B^T at any 2-byte alignment, any K
+    if (tail && (es == 2 || (a_aligned && (a->stride_bn * es) % 16 == 0)) && a->stride_am >= a->k && a->stride_bn >= a->k) {
+      *tail = true;
+      return 2;
+    }
   }
   return 0;
 }

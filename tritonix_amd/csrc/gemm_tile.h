@@ -955,7 +955,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // no multiple of BK, rows that are not 16-byte aligned or an N that ends inside a chunk, the host sets tail_slab
   // and the last slab of the K range (the only one whose chunks can cross the end of a row of A, or the end of the
   // last row of B) is left out of the ring and loaded element by element, zero-filled, after the K loop.
-  const bool tail_here = FAST && !PERSIST && !BT && !CONV && p.tail_slab != 0 && kt1 == kt_total && kt1 > kt0;
+  const bool tail_here = FAST && !PERSIST && !CONV && p.tail_slab != 0 && kt1 == kt_total && kt1 > kt0;
   const int KT = kt1 > kt0 ? kt1 - kt0 - (tail_here ? 1 : 0) : 0;          // slabs of this workgroup in the ring (per tile)
 
   // ---- the tile the loader works on: origin, DMA bases and per-lane byte offsets.
@@ -1101,6 +1101,25 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       }
       *TNX_LDS(i32x4, stage_base + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
     }
+    if constexpr (BT) {
+      // k-contiguous B: the slab holds BN rows of B^T, chunked and swizzled like the A slab
+      for (int idx = t0; idx < BN * C::CPR_A; idx += C::THREADS) {
+        const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
+        const int64_t gn = n0 + row, gk = k0 + cs * EPC;
+        i32x4 v = {0, 0, 0, 0};
+        if (gn < p.n && gk < p.k) {
+          if (p.sbk == 1 && gk + EPC <= p.k) {
+            v = *(const chunk_t*)(bp + gn * p.sbn + gk);
+          } else {
+            elem_t e[EPC];
+#pragma unroll
+            for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? bp[gn * p.sbn + (gk + x) * p.sbk] : (elem_t)0;
+            __builtin_memcpy(&v, e, 16);
+          }
+        }
+        *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
+      }
+    } else
     for (int idx = t0; idx < BK * C::CPR_B; idx += C::THREADS) {
       const int row = idx / C::CPR_B, cs = idx % C::CPR_B;
       const int64_t gk = k0 + row, gn = n0 + cs * EPC;
@@ -1606,7 +1625,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     }
     TNX_PHASE(1);
     k_loop();
-    if constexpr (FAST && !BT && !CONV) {
+    if constexpr (FAST && !CONV) {
       if (tail_here) {
         // the left-out slab: every wave is done with the ring, slot 0 takes it, one slab of MFMAs follows
         __syncthreads();
