@@ -122,9 +122,9 @@ typedef struct tnx_gemm_args {
  * Which loader moves the operands follows from their layout, not from an argument:
  *   - A row-major (stride_ak == 1) and B row-major (stride_bn == 1): the direct-to-LDS loader of every built tile.
  *     With K a multiple of block_k, 16-byte aligned rows and base pointers and N a multiple of 16 bytes of elements
- *     every K slab goes through it; otherwise (16-bit types: any 2-byte-aligned rows and pointers, any K and N;
- *     int8: rows and pointers still 16-byte aligned, any K and N; row pitches at least the row length) the last K
- *     slab is loaded element by element with zero fill and the slabs before it through the direct loader.
+ *     every K slab goes through it; otherwise (rows and pointers at the element's own alignment, any K and N, row
+ *     pitches at least the row length) the last K slab is loaded chunk by chunk with zero fill and the slabs
+ *     before it through the direct loader.
  *     TNX_SCHED_PERSISTENT takes the first form only.
  *   - A row-major and B k-contiguous (stride_bk == 1, the view w.t() of a row-major weight): a direct-to-LDS loader
  *     of its own, in the tiles whose K slab is 128 bytes per row, under the same two sets of conditions (K a multiple

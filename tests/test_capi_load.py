@@ -85,7 +85,7 @@ def test_supported_status_codes_and_python_exceptions():
 def test_ragged_layouts_need_a_generic_kernel():
     lib = _C.load()
     # row-major 16-bit operands with a ragged K, rows that are not 16-byte aligned or a ragged N: every tile takes
-    # them (DMA loader, last K slab element-wise); the persistent schedule and int8 rows off 16 bytes do not
+    # them (DMA loader, last K slab chunk by chunk), int8 included; the persistent schedule does not
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500))) == _C.OK          # 128x128x64 w4 s2
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500, num_stages=3))) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(args(n=509, stride_bk=509, stride_cm=509, num_stages=3))) == _C.OK
@@ -93,7 +93,7 @@ def test_ragged_layouts_need_a_generic_kernel():
                                                     schedule=_C.SCHED_PERSISTENT))) == _C.E_UNSUPPORTED
     i8 = dict(in_dtype=_C.I8, out_dtype=_C.I32, block_k=128, num_stages=3)
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=528, stride_am=528, **i8))) == _C.OK       # ragged K, aligned rows
-    assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500, **i8))) == _C.E_UNSUPPORTED
+    assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=500, **i8))) == _C.OK
     assert lib.tnx_gemm_supported(ctypes.byref(args(k=500, stride_am=400, num_stages=3))) == _C.E_UNSUPPORTED   # rows overlap
     # k-contiguous B (w.t() of a row-major weight) has a DMA loader of its own in every tile whose K slab is 128 bytes
     # per row, 16-bit rows at any alignment included

@@ -81,7 +81,7 @@ static int check_common(const tnx_gemm_args* a) {
 // 16-byte aligned rows and base pointers and k % block_k == 0.
 // 0: element-wise loader; 1: DMA loader, A and B row-major; 2: DMA loader, B k-contiguous.
 // *tail (layout 1 only): the operands are row-major but not as the DMA loader likes them best -- K no multiple of
-// block_k, rows or base pointers of 16-bit operands not 16-byte aligned (the loads take any 2-byte-aligned address),
+// block_k, rows or base pointers not 16-byte aligned (the loads take any byte address: probed on the hardware),
 // N ending inside a 16-byte chunk -- so the last K slab, the only one whose chunks can cross the end of a row of A
 // or of the last row of B, is loaded element by element instead (GemmParams::tail_slab).
 static int dma_layout(const tnx_gemm_args* a, bool* tail = nullptr) {
@@ -96,9 +96,7 @@ static int dma_layout(const tnx_gemm_args* a, bool* tail = nullptr) {
       (int64_t)a->block_k * a->stride_bk * es + (int64_t)a->block_n * es < (1ll << 32)) {
     const bool strict = a_aligned && a->k % a->block_k == 0 && (a->stride_bk * es) % 16 == 0 && a->n % vec == 0 && a->n >= vec;
     if (strict) return 1;
-    // int8 operands keep 16-byte aligned rows (1-byte-aligned DMA addresses are untried); only K and N may be ragged
-    const bool loose_ok = tail && (es == 2 || (a_aligned && (a->stride_bk * es) % 16 == 0)) && a->stride_am >= a->k &&
-                          a->stride_bk >= a->n;
+    const bool loose_ok = tail && a->stride_am >= a->k && a->stride_bk >= a->n;
     if (loose_ok) {
       *tail = true;
       return 1;
@@ -106,8 +104,8 @@ static int dma_layout(const tnx_gemm_args* a, bool* tail = nullptr) {
   }
   if (a->stride_bk == 1 && a->stride_bn >= 0 && (int64_t)a->block_n * a->stride_bn * es + (int64_t)a->block_k * es < (1ll << 32)) {
     if (a_aligned && a->k % a->block_k == 0 && (a->stride_bn * es) % 16 == 0) return 2;
-    // the same relaxation for a k-contiguous B: rows of B^T at any 2-byte alignment, any K
-    if (tail && (es == 2 || (a_aligned && (a->stride_bn * es) % 16 == 0)) && a->stride_am >= a->k && a->stride_bn >= a->k) {
+    // the same relaxation for a k-contiguous B: rows of B^T at any alignment, any K
+    if (tail && a->stride_am >= a->k && a->stride_bn >= a->k) {
       *tail = true;
       return 2;
     }

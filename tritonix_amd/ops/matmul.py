@@ -181,24 +181,13 @@ def dma_layout(a, b) -> int:
     layouts the direct-to-LDS loaders take as they are; 3, 4 = the same two layouts as they take them with the last K
     slab loaded chunk by chunk (ragged K, rows off 16 bytes); 0 = anything else (the two tiles built with the element-wise loader)."""
     es = a.element_size()
-    if not (a.stride(1) == 1 and a.stride(0) >= 0 and (a.stride(0) * es) % 16 == 0
-            and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0):
-        # 3 / 4 = the same two layouts of 16-bit operands at any 2-byte alignment: the DMA loader with a last K slab
-        # that is loaded chunk by chunk
-        if es == 2 and a.stride(1) == 1 and a.stride(0) >= a.shape[1]:
-            if b.stride(1) == 1 and b.stride(0) >= b.shape[1]:
-                return 3
-            if b.stride(0) == 1 and b.stride(1) >= b.shape[0]:
-                return 4
+    if not (a.stride(1) == 1 and a.stride(0) >= a.shape[1]):
         return 0
-    if b.stride(1) == 1 and b.stride(0) >= 0 and (b.stride(0) * es) % 16 == 0 and b.shape[1] % (16 // es) == 0:
-        return 1
-    if b.stride(1) == 1 and b.stride(0) >= b.shape[1] and (es == 2 or (b.stride(0) * es) % 16 == 0):
-        return 3
-    if b.stride(0) == 1 and b.stride(1) >= 0 and (b.stride(1) * es) % 16 == 0:
-        return 2
-    if b.stride(0) == 1 and b.stride(1) >= b.shape[0] and es == 2:
-        return 4
+    aligned = (a.stride(0) * es) % 16 == 0 and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0
+    if b.stride(1) == 1 and b.stride(0) >= b.shape[1]:
+        return 1 if aligned and (b.stride(0) * es) % 16 == 0 and b.shape[1] % (16 // es) == 0 else 3
+    if b.stride(0) == 1 and b.stride(1) >= b.shape[0]:
+        return 2 if aligned and (b.stride(1) * es) % 16 == 0 else 4
     return 0
 
 
