@@ -44,7 +44,7 @@ NOMINAL_SCLK_MHZ = 2400.0
 # L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # (KiB per dispatch), each scaled by what the same counter reads for this file's 2^28-byte calibration pass.
 # The two readings and the two factors are in profiles/gemm_tile_c2_clock_power_counters.md (section 4).
-TRAFFIC_KIB_C2 = {"fetch": 788932.5, "fetch_scale": 2.0, "write": 187410.2, "write_scale": 1.0}
+TRAFFIC_KIB_C2 = {"fetch": 788937.5, "fetch_scale": 2.0, "write": 187422.1, "write_scale": 1.0}
 TRAFFIC_BYTES_C2 = int((TRAFFIC_KIB_C2["fetch"] * TRAFFIC_KIB_C2["fetch_scale"]
                         + TRAFFIC_KIB_C2["write"] * TRAFFIC_KIB_C2["write_scale"]) * 1024)
 
