@@ -402,3 +402,39 @@ def test_k_contiguous_b_takes_its_own_dma_loader(device, dtype, tile, shape):
         check_fp(out, ref)
     # the same products in the same order as with a row-major copy of B
     assert torch.equal(out, gemm(ad, b.contiguous(), cfg(*tile, **extra), kernel=kernel))
+
+
+# ---- operands beyond 4 GiB and 2^31 elements: every byte offset is 64-bit -----------------------
+@pytest.mark.parametrize("shape", [(49152, 49152, 49152), (50000, 49160, 49200)], ids=lambda s: "x".join(map(str, s)))
+def test_operands_beyond_four_gibibytes(device, shape):
+    """A, B and C of 4.8 GB each (the second case ragged, rows off 16 bytes).  No CPU product of that size: row sums
+    C.1 == A.(B.1) and column sums 1.C == (1.A).B in float64 on the GPU (chunked reductions), and the far corner of
+    C element by element.  The bounds are those of whole_matrix_identity: many times the 16-bit output rounding,
+    far below what a tile written to the wrong place would move."""
+    m, n, k = shape
+    torch.manual_seed(0)
+    a = torch.empty((m, k), device=device, dtype=torch.bfloat16)
+    b = torch.empty((k, n), device=device, dtype=torch.bfloat16)
+    for i in range(0, m, 4096):
+        a[i:i + 4096] = (torch.randn(min(4096, m - i), k, device=device) / k ** 0.5).bfloat16()
+    for i in range(0, k, 4096):
+        b[i:i + 4096] = torch.randn(min(4096, k - i), n, device=device).bfloat16()
+    c = gemm(a, b, cfg(256, 256, 64, 4, 2, superblock=1))
+    b1 = torch.cat([b[i:i + 4096].sum(dim=1, dtype=torch.float64) for i in range(0, k, 4096)])
+    rows = torch.cat([c[i:i + 2048].sum(dim=1, dtype=torch.float64) for i in range(0, m, 2048)])
+    want_rows = torch.cat([a[i:i + 2048].double() @ b1 for i in range(0, m, 2048)])
+    assert float((rows - want_rows).abs().max() / want_rows.abs().max()) < 4e-3
+    a1 = torch.zeros(k, device=device, dtype=torch.float64)
+    cols = torch.zeros(n, device=device, dtype=torch.float64)
+    for i in range(0, m, 2048):
+        a1 += a[i:i + 2048].sum(dim=0, dtype=torch.float64)
+        cols += c[i:i + 2048].sum(dim=0, dtype=torch.float64)
+    want_cols = torch.zeros(n, device=device, dtype=torch.float64)
+    for i in range(0, k, 2048):
+        want_cols += a1[i:i + 2048] @ b[i:i + 2048].double()
+    assert float((cols - want_cols).abs().max() / want_cols.abs().max()) < 4e-3
+    idx = torch.tensor([0, 1, m // 2, m - 2, m - 1], device=device)
+    corner = a[idx].float() @ b[:, n - 64:].float()
+    assert float((c[idx][:, n - 64:].float() - corner).abs().max() / corner.abs().max()) < 1e-2
+    del a, b, c
+    torch.cuda.empty_cache()
