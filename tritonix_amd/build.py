@@ -74,10 +74,11 @@ def parse_only(spec):
     out = []
     for item in spec.split(","):
         dt, *nums = item.strip().split(":")
-        bm, bn, bk, nw, st = (int(v) for v in nums)
+        generic = nums[-1] == "generic"          # ...:generic also builds the tile with the chunk-wise loader
+        bm, bn, bk, nw, st = (int(v) for v in (nums[:-1] if generic else nums))
         if not tile_valid(TAGS[dt][1], bm, bn, bk, nw, st):
             raise SystemExit(f"{item}: not a buildable tile")
-        out.append((dt, bm, bn, bk, nw, st, False))
+        out.append((dt, bm, bn, bk, nw, st, generic))
     return out
 
 

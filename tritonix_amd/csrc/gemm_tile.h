@@ -1078,64 +1078,96 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // kernels built without the DMA loader and for the left-out last slab of a tail_slab launch.
   // (t0: the thread's index in the workgroup, handed in so that the DMA kernels need not keep threadIdx.x alive
   // across their K loop for the one call after it)
-  auto load_slab_generic = [&](int kt_global, uint32_t stage_base, int t0) __attribute__((always_inline)) {
-    typedef typename std::conditional<ES == 2, uint16_t, uint8_t>::type elem_t;
-    typedef typename std::conditional<ES == 2, i32x4_loose, i32x4_bytes>::type chunk_t;
-    constexpr int EPC = 16 / ES;                         // elements per chunk
+  // The loader in two halves, so that the kernels built without the DMA loader can fetch slab t + STAGES into
+  // registers before the MFMAs of a period and put it into LDS after them (gen_fetch, gen_store).
+  constexpr int GEN_B_ROWS = BT ? BN : BK, GEN_B_CPR = BT ? C::CPR_A : C::CPR_B;
+  constexpr int GEN_NA = (BM * C::CPR_A + C::THREADS - 1) / C::THREADS;
+  constexpr int GEN_NB = (GEN_B_ROWS * GEN_B_CPR + C::THREADS - 1) / C::THREADS;
+  typedef typename std::conditional<ES == 2, uint16_t, uint8_t>::type gen_elem_t;
+  typedef typename std::conditional<ES == 2, i32x4_loose, i32x4_bytes>::type gen_chunk_t;
+  constexpr int EPC = 16 / ES;                           // elements per chunk
+  // chunk idx of the A part of slab kt_global: row idx / CPR_A, k chunk idx % CPR_A
+  auto gen_fetch_a = [&](int kt_global, int idx) __attribute__((always_inline)) -> i32x4 {
+    const gen_elem_t* ap = (const gen_elem_t*)p.a;
+    const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
+    const int64_t gm = m0 + row, gk = (int64_t)kt_global * BK + cs * EPC;
+    i32x4 v = {0, 0, 0, 0};
+    if (idx < BM * C::CPR_A && gm < p.m && gk < p.k) {
+      if (p.sak == 1 && gk + EPC <= p.k) {
+        v = *(const gen_chunk_t*)(ap + gm * p.sam + gk);
+      } else {
+        gen_elem_t e[EPC];
+#pragma unroll
+        for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? ap[gm * p.sam + (gk + x) * p.sak] : (gen_elem_t)0;
+        __builtin_memcpy(&v, e, 16);
+      }
+    }
+    return v;
+  };
+  // chunk idx of the B part: k row idx / CPR_B, column chunk idx % CPR_B -- or, for the k-contiguous-B kernels, whose
+  // slab holds BN rows of B^T chunked and swizzled like the A slab, column idx / CPR_A, k chunk idx % CPR_A
+  auto gen_fetch_b = [&](int kt_global, int idx) __attribute__((always_inline)) -> i32x4 {
+    const gen_elem_t* bp = (const gen_elem_t*)p.b;
+    const int row = idx / GEN_B_CPR, cs = idx % GEN_B_CPR;
     const int64_t k0 = (int64_t)kt_global * BK;
-    const elem_t* ap = (const elem_t*)p.a;
-    const elem_t* bp = (const elem_t*)p.b;
-    for (int idx = t0; idx < BM * C::CPR_A; idx += C::THREADS) {
-      const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
-      const int64_t gm = m0 + row, gk = k0 + cs * EPC;
-      i32x4 v = {0, 0, 0, 0};
-      if (gm < p.m && gk < p.k) {
-        if (p.sak == 1 && gk + EPC <= p.k) {
-          v = *(const chunk_t*)(ap + gm * p.sam + gk);
-        } else {
-          elem_t e[EPC];
-#pragma unroll
-          for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? ap[gm * p.sam + (gk + x) * p.sak] : (elem_t)0;
-          __builtin_memcpy(&v, e, 16);
-        }
-      }
-      *TNX_LDS(i32x4, stage_base + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
-    }
+    i32x4 v = {0, 0, 0, 0};
     if constexpr (BT) {
-      // k-contiguous B: the slab holds BN rows of B^T, chunked and swizzled like the A slab
-      for (int idx = t0; idx < BN * C::CPR_A; idx += C::THREADS) {
-        const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
-        const int64_t gn = n0 + row, gk = k0 + cs * EPC;
-        i32x4 v = {0, 0, 0, 0};
-        if (gn < p.n && gk < p.k) {
-          if (p.sbk == 1 && gk + EPC <= p.k) {
-            v = *(const chunk_t*)(bp + gn * p.sbn + gk);
-          } else {
-            elem_t e[EPC];
-#pragma unroll
-            for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? bp[gn * p.sbn + (gk + x) * p.sbk] : (elem_t)0;
-            __builtin_memcpy(&v, e, 16);
-          }
-        }
-        *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
-      }
-    } else
-    for (int idx = t0; idx < BK * C::CPR_B; idx += C::THREADS) {
-      const int row = idx / C::CPR_B, cs = idx % C::CPR_B;
-      const int64_t gk = k0 + row, gn = n0 + cs * EPC;
-      i32x4 v = {0, 0, 0, 0};
-      if (gk < p.k && gn < p.n) {
-        if (p.sbn == 1 && gn + EPC <= p.n) {
-          v = *(const chunk_t*)(bp + gk * p.sbk + gn);
+      const int64_t gn = n0 + row, gk = k0 + cs * EPC;
+      if (idx < GEN_B_ROWS * GEN_B_CPR && gn < p.n && gk < p.k) {
+        if (p.sbk == 1 && gk + EPC <= p.k) {
+          v = *(const gen_chunk_t*)(bp + gn * p.sbn + gk);
         } else {
-          elem_t e[EPC];
+          gen_elem_t e[EPC];
 #pragma unroll
-          for (int x = 0; x < EPC; ++x) e[x] = gn + x < p.n ? bp[gk * p.sbk + (gn + x) * p.sbn] : (elem_t)0;
+          for (int x = 0; x < EPC; ++x) e[x] = gk + x < p.k ? bp[gn * p.sbn + (gk + x) * p.sbk] : (gen_elem_t)0;
           __builtin_memcpy(&v, e, 16);
         }
       }
-      *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_B + ((cs ^ C::swzB(row)) << 4)) = v;
+    } else {
+      const int64_t gk = k0 + row, gn = n0 + cs * EPC;
+      if (idx < GEN_B_ROWS * GEN_B_CPR && gk < p.k && gn < p.n) {
+        if (p.sbn == 1 && gn + EPC <= p.n) {
+          v = *(const gen_chunk_t*)(bp + gk * p.sbk + gn);
+        } else {
+          gen_elem_t e[EPC];
+#pragma unroll
+          for (int x = 0; x < EPC; ++x) e[x] = gn + x < p.n ? bp[gk * p.sbk + (gn + x) * p.sbn] : (gen_elem_t)0;
+          __builtin_memcpy(&v, e, 16);
+        }
+      }
     }
+    return v;
+  };
+  auto gen_store_a = [&](uint32_t stage_base, int idx, i32x4 v) __attribute__((always_inline)) {
+    const int row = idx / C::CPR_A, cs = idx % C::CPR_A;
+    if (idx < BM * C::CPR_A) *TNX_LDS(i32x4, stage_base + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
+  };
+  auto gen_store_b = [&](uint32_t stage_base, int idx, i32x4 v) __attribute__((always_inline)) {
+    const int row = idx / GEN_B_CPR, cs = idx % GEN_B_CPR;
+    if (idx < GEN_B_ROWS * GEN_B_CPR) {
+      if constexpr (BT) *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_A + ((cs ^ C::swzA(row)) << 4)) = v;
+      else *TNX_LDS(i32x4, stage_base + C::A_BYTES + row * C::ROWB_B + ((cs ^ C::swzB(row)) << 4)) = v;
+    }
+  };
+  auto gen_fetch = [&](int kt_global, int t0, i32x4 (&ra)[GEN_NA], i32x4 (&rb)[GEN_NB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < GEN_NA; ++u) ra[u] = gen_fetch_a(kt_global, t0 + u * C::THREADS);
+#pragma unroll
+    for (int u = 0; u < GEN_NB; ++u) rb[u] = gen_fetch_b(kt_global, t0 + u * C::THREADS);
+  };
+  auto gen_store = [&](uint32_t stage_base, int t0, const i32x4 (&ra)[GEN_NA], const i32x4 (&rb)[GEN_NB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < GEN_NA; ++u) gen_store_a(stage_base, t0 + u * C::THREADS, ra[u]);
+#pragma unroll
+    for (int u = 0; u < GEN_NB; ++u) gen_store_b(stage_base, t0 + u * C::THREADS, rb[u]);
+  };
+  // one chunk at a time: for the prologue of the kernels without the DMA loader and the one call after the K loop
+  // of a tail_slab launch, where nothing is there to overlap with and registers are better left alone
+  auto load_slab_generic = [&](int kt_global, uint32_t stage_base, int t0) __attribute__((always_inline)) {
+#pragma unroll 1
+    for (int idx = t0; idx < BM * C::CPR_A; idx += C::THREADS) gen_store_a(stage_base, idx, gen_fetch_a(kt_global, idx));
+#pragma unroll 1
+    for (int idx = t0; idx < GEN_B_ROWS * GEN_B_CPR; idx += C::THREADS) gen_store_b(stage_base, idx, gen_fetch_b(kt_global, idx));
   };
 
   // CONV: the first 64 threads write the taps of the next slab to tabulate into the table of its parity and move
@@ -1589,15 +1621,20 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
     conv_period_begin();
     const uint32_t dst = stage_of(t);
-    if constexpr (!FAST) load_slab_generic(kt0 + t + STAGES, dst, tid);
     const uint32_t sa1 = stage_of(t + 1), sb1 = sa1 + C::A_BYTES;
     if constexpr (FAST) {
       last_step(sa1, sb1, Yes{}, dst, Par0{}, Yes{});
       inner_steps(sa1, sb1, Yes{}, dst, Par0{});
       dma_advance();
     } else {
+      // slab t + STAGES: fetched into registers now, written to the freed slot after this period's MFMAs; the
+      // writes have to be in LDS before the next barrier lets anyone read them
+      i32x4 ra[GEN_NA], rb[GEN_NB];
+      gen_fetch(kt0 + t + STAGES, tid, ra, rb);
       last_step(sa1, sb1, No{}, 0u, Par0{}, Yes{});
       inner_steps(sa1, sb1, No{}, 0u, Par0{});
+      gen_store(dst, tid, ra, rb);
+      __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
     }
   }
   // (2) ring draining: nothing left to issue
