@@ -181,8 +181,14 @@ def generate(instances):
     for inst in instances:
         groups.setdefault((inst[0], inst[1], inst[2]), []).append(inst)
     files, names = [], []
-    for (dt, bm, bn), items in sorted(groups.items()):
-        name = f"inst_{dt}_m{bm}_n{bn}"
+    # at most three kernels per translation unit, the largest tiles first: the biggest unit used to take four
+    # minutes on its own and set the wall time of the whole build
+    parts = []
+    for (dt, bm, bn), items in sorted(groups.items(), key=lambda kv: -kv[0][1] * kv[0][2]):
+        for c in range(0, len(items), 3):
+            suffix = f"_p{c // 3}" if len(items) > 3 else ""
+            parts.append(((dt, bm, bn), f"inst_{dt}_m{bm}_n{bn}{suffix}", items[c:c + 3]))
+    for (dt, bm, bn), name, items in parts:
         tag = TAGS[dt][0]
         rows = ",\n".join(
             f"    TNX_ENTRY({tag}, {i[1]}, {i[2]}, {i[3]}, {i[4]}, {i[5]}, {'true' if i[6] else 'false'})" for i in items)
