@@ -221,15 +221,20 @@ def test_memoised_config_follows_the_operand_layout(device, monkeypatch):
     a_off.copy_(ad)
     assert mm.dma_layout(a_off, b_contig) == 3 and mm.dma_layout(ad, b_contig) == 1 and mm.dma_layout(ad, wd.t()) == 2
     assert torch.equal(tritonix_amd.triton_matmul(a_off, b_contig), out1)
-    # a column-major A is none of the DMA layouts: the two tiles built with the element-wise loader
+    # a column-major A is none of the DMA layouts: the wrapper hands the kernel a row-major copy (same bits as out1),
+    # the kernel object itself takes the strides as they are (one of the two tiles built with the chunk-wise loader)
     a_cm = ad.t().contiguous().t()
     assert a_cm.stride() == (1, 512) and mm.dma_layout(a_cm, b_contig) == 0
-    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_cm, b_contig), ref)[0]
-    # a memo entry the engine refuses for these operands is replaced, not raised
-    mm._matmul_cfg[(512, 384, 256, torch.float16, 0)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, 1)],
-                                                             block_m=256, block_n=256, num_stages=2, num_warps=4)
-    assert oracle.within_tolerance(tritonix_amd.triton_matmul(a_cm, b_contig), ref)[0]
-    assert mm._matmul_cfg[(512, 384, 256, torch.float16, 0)]["block_m"] == 128       # replaced by the built-in choice
+    assert torch.equal(tritonix_amd.triton_matmul(a_cm, b_contig), out1)
+    assert mm.dma_operands(a_cm, b_contig)[0].stride() == (256, 1)
+    raw = mm._launch_matmul(a_cm, b_contig, dict(block_m=128, block_n=128, block_k=64, group_m=8, num_stages=2, num_warps=4))
+    assert oracle.within_tolerance(raw, ref)[0]
+    # a memo entry the engine refuses for these operands is replaced, not raised: the persistent schedule does not
+    # take operands off 16 bytes
+    mm._matmul_cfg[(512, 384, 256, torch.float16, 3)] = dict(mm._matmul_cfg[(512, 384, 256, torch.float16, 3)],
+                                                             block_m=128, block_n=128, num_stages=3, num_warps=4, persistent=1)
+    assert torch.equal(tritonix_amd.triton_matmul(a_off, b_contig), out1)
+    assert "persistent" not in mm._matmul_cfg[(512, 384, 256, torch.float16, 3)]      # replaced by the built-in choice
     mm._matmul_cfg.clear()
 
 

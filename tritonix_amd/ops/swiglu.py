@@ -74,6 +74,7 @@ def glu(x: torch.Tensor, w12: torch.Tensor, activation: str = "silu") -> torch.T
         raise ValueError("the interleaved weight must have an even number of columns")
     if x.dtype not in (torch.float16, torch.bfloat16):
         raise ValueError(f"glu is built for float16 and bfloat16, got {x.dtype}")
+    x, w12 = _mm.dma_operands(x, w12)
     m, k = x.shape
     n = w12.shape[1]
     key = (m, n, k, x.dtype, _mm.dma_layout(x, w12))
