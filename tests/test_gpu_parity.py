@@ -131,6 +131,29 @@ def test_c4_glu_scaled(device, activation, config):
     check_fp(z, oracle.reference_glu(x, w12, activation))
 
 
+@pytest.mark.parametrize("activation", ["silu", "sigmoid"])
+@pytest.mark.parametrize("config", [cfg(256, 256, 64, 8, 2), cfg(128, 128, 64, 4, 3)],
+                         ids=lambda c: "x".join(str(v) for v in c.values()))
+def test_glu_ragged_operands_on_the_dma_path(device, activation, config):
+    """K no multiple of block_k, rows of x and of the interleaved weight off 16 bytes, a gated width that ends inside a
+    chunk: the last K slab is loaded chunk by chunk.  Same bits as the launch on zero-padded, aligned copies."""
+    g = torch.Generator("cpu").manual_seed(77)
+    m, k, n2 = 700, 1030, 2 * 1301
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w12 = (0.05 * torch.randn(k, n2, generator=g)).bfloat16()
+    z = torch.full((m, n2 // 2), 7, device=device, dtype=torch.bfloat16)
+    run(glu_kernel, x.to(device), w12.to(device), z, config, activation=activation)
+    check_fp(z, oracle.reference_glu(x, w12, activation))
+    kp, np2 = 1088, 2 * 1304
+    xp = torch.zeros((m, kp), dtype=torch.bfloat16)
+    wp = torch.zeros((kp, np2), dtype=torch.bfloat16)
+    xp[:, :k] = x
+    wp[:k, :n2] = w12
+    zp = torch.full((m, np2 // 2), 7, device=device, dtype=torch.bfloat16)
+    run(glu_kernel, xp.to(device), wp.to(device), zp, config, activation=activation)
+    assert torch.equal(z, zp[:, :n2 // 2])
+
+
 def test_c4_glu_full_size_rows(device):
     x, w12 = oracle.make_inputs("C4")
     xd, wd = x.to(device), w12.to(device)
