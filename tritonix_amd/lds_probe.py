@@ -1,8 +1,8 @@
 """LDS bank conflicts of the address patterns the tile kernels use, and which lanes an LDS instruction serves together.
 
     rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_INSTS_LDS --kernel-trace --output-format csv \\
-        -d gpurun_out/lds_probe -o p -- python3 -m tritonix_amd.lds_probe
-    python3 -m tritonix_amd.lds_probe --counters gpurun_out/lds_probe/<...>/p_counter_collection.csv
+        -d /tmp/lds_probe -o p -- python3 -m tritonix_amd.lds_probe
+    python3 -m tritonix_amd.lds_probe --counters /tmp/lds_probe/<host>/p_counter_collection.csv
 
 The first command launches ``tnx_probe_lds`` once per pattern below (one wave, 16000 instructions each); the second
 reads the counters of those dispatches, in order, and prints conflict and active cycles per instruction.  The
