@@ -23,6 +23,8 @@ Switches for profiling and for the clock / power evidence:
   --splitk-reduce atomic   C3 with the K slices added by fp32 atomics instead of the ordered hand-over (for the A/B)
   --mfma-ceiling     time tnx_probe_mfma: nothing but MFMAs on register operands, 16x16 and 32x32 tiles, random and
                      all-zero operands; what the pipes sustain on this board before any data is moved ("mfma_ceiling")
+  --shape-sweep      the built-in tile choice on a ladder of other bf16 shapes (GEMV to 4096^3, aligned and ragged)
+                     beside the vendor library's GEMM on the same operands ("shape_sweep")
   --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
                      socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
@@ -63,6 +65,9 @@ def parse():
                     help="C3 only: how the K slices meet (ordered = stored apart, summed in slice order; atomic = fp32 atomic adds)")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="also time the MFMA-only loop (no data movement) for both MFMA shapes and both operand kinds")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="also time the built-in tile choice on a ladder of other bf16 shapes (GEMV to 2048^3, aligned "
+                         "and ragged) beside the vendor library's GEMM on the same operands (\"shape_sweep\")")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -188,6 +193,37 @@ def sustain(step, seconds, flops):
     return out
 
 
+SWEEP_SHAPES = [(1, 4096, 4096), (8, 14336, 4096), (32, 4096, 14336), (64, 8192, 8192), (128, 8192, 8192),
+                (512, 4096, 4096), (1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096),
+                (4096, 4096, 4104), (4096, 4100, 4096), (4100, 4096, 4096)]
+
+
+def shape_sweep(torch, dev, mm):
+    """Kernel time of the built-in configuration (`tnx_gemm_default_config`) on other shapes, launches bound once
+    (`prepare`), B rotated over several copies so that skinny shapes stream it from HBM; the vendor's GEMM on the
+    same operands beside it."""
+    rows = []
+    for m, n, k in SWEEP_SHAPES:
+        g = torch.Generator("cpu").manual_seed(m + n + k)
+        a = (torch.randn(m, k, generator=g) / k ** 0.5).bfloat16().to(dev)
+        b0 = torch.randn(k, n, generator=g).bfloat16()
+        bs = [b0.to(dev).clone() for _ in range(4 if k * n * 2 < 300e6 else 2)]
+        cfg = mm.default_config(a, bs[0])
+        kern = mm.gemm_splitk_kernel if cfg.get("split_k", 1) > 1 else mm.matmul_kernel
+        c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
+        ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), 1, n, 1, **cfg) for b in bs]
+        for i in range(20):
+            ls[i % len(ls)]()
+        ours = region_time(lambda i: ls[i % len(ls)](), 50)
+        for i in range(10):
+            torch.matmul(a, bs[i % len(bs)], out=c)
+        vendor = region_time(lambda i: torch.matmul(a, bs[i % len(bs)], out=c), 50)
+        rows.append({"shape": [m, n, k], "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),
+                     "gbs": round(2.0 * (m * k + k * n + m * n) / ours / 1e6, 1), "vendor_ms": round(vendor, 4),
+                     "config": cfg})
+    return rows
+
+
 def mfma_ceiling(torch, dev, dtype_code, peak):
     """T(FL)OP/s of the MFMA-only loop: {"16x16": {"random": .., "zeros": ..}, "32x32": {...}} (same protocol as the
     kernels: pre-roll, then one HIP-event pair around back-to-back launches on the launch stream)."""
@@ -277,6 +313,8 @@ def main():
     if args.mfma_ceiling:
         out["mfma_ceiling"] = {"bf16": mfma_ceiling(torch, dev, _C.BF16, PEAK["bf16"]),
                                "i8": mfma_ceiling(torch, dev, _C.I8, PEAK["i8"])}
+    if args.shape_sweep:
+        out["shape_sweep"] = shape_sweep(torch, dev, mm)
     extras_wanted = [s for s in only if s != "C2"]
     if extras_wanted:
         out["per_config"] = extras(torch, dev, oracle, mm, sg, args, operands, extras_wanted)
