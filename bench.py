@@ -25,6 +25,8 @@ Switches for profiling and for the clock / power evidence:
                      all-zero operands; what the pipes sustain on this board before any data is moved ("mfma_ceiling")
   --shape-sweep      the built-in tile choice on a ladder of other bf16 shapes (GEMV to 4096^3, aligned and ragged)
                      beside the vendor library's GEMM on the same operands ("shape_sweep")
+  --conv1x1-sweep    the 1x1 layers of a ResNet-50 (bf16, batch 8 / 32 / 128) on the GEMM route and on the conv2d
+                     kernel the library would otherwise take, built-in tiles both, beside MIOpen ("conv1x1_sweep")
   --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
                      socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
@@ -68,6 +70,8 @@ def parse():
     ap.add_argument("--shape-sweep", action="store_true",
                     help="also time the built-in tile choice on a ladder of other bf16 shapes (GEMV to 2048^3, aligned "
                          "and ragged) beside the vendor library's GEMM on the same operands (\"shape_sweep\")")
+    ap.add_argument("--conv1x1-sweep", action="store_true",
+                    help="also time ResNet-50's 1x1 layers on the GEMM route and on the conv2d kernels (\"conv1x1_sweep\")")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -224,6 +228,64 @@ def shape_sweep(torch, dev, mm):
     return rows
 
 
+# c_in, plane side, c_out of the 1x1 layers of a ResNet-50 (unit stride: the projections inside the bottleneck blocks)
+CONV1X1_LAYERS = [(64, 56, 256), (256, 56, 64), (256, 56, 128), (256, 56, 512), (512, 28, 128), (128, 28, 512),
+                  (512, 28, 1024), (1024, 14, 256), (256, 14, 1024), (1024, 14, 2048), (2048, 7, 512), (512, 7, 2048)]
+
+
+def conv1x1_sweep(torch, dev):
+    """Kernel time of the 1x1 layers with the library's own tile: the GEMM route (LOADER="gemm"), the conv2d kernel
+    "auto" would take without that route (direct-to-LDS where it applies, else register-staged), what "auto" takes,
+    and the vendor's conv2d on the same tensors.  Launches bound once (`prepare`)."""
+    import ctypes
+
+    from tritonix_amd import _C
+    from tritonix_amd.ops.conv2d import forward as conv
+
+    rows = []
+    zero = dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0, GROUP_SIZE_M=8)
+    for batch in (8, 32, 128):
+        for c_in, hw, c_out in CONV1X1_LAYERS:
+            g = torch.Generator("cpu").manual_seed(batch + c_in + hw)
+            x = torch.randn(batch, c_in, hw, hw, generator=g).bfloat16().to(dev)
+            w = (torch.randn(c_out, c_in, 1, 1, generator=g) / c_in ** 0.5).bfloat16().to(dev)
+            bias = torch.randn(c_out, generator=g).bfloat16().to(dev)
+            y = torch.empty(batch, c_out, hw, hw, device=dev, dtype=torch.bfloat16)
+
+            def bound(loader):
+                return conv.conv2d_forward_kernel.prepare(y, x, w, bias, batch, c_in, hw, hw, c_out, hw, hw, 1, 1, 1, 1, 0, 0,
+                                                          1, 1, batch * hw * hw, c_out, c_in, LOADER=loader, **zero)
+
+            def timed(fn):
+                for _ in range(20):
+                    fn()
+                return region_time(lambda i: fn(), 50)
+
+            other, other_name = bound("dma"), "dma"
+            if _C.load().tnx_conv2d_supported(ctypes.byref(other.args)) != _C.OK:
+                other, other_name = bound("registers"), "registers"
+            auto = bound("auto")
+            row = {"batch": batch, "layer": [c_in, hw, c_out], "gemm_us": round(timed(bound("gemm")) * 1e3, 1),
+                   "conv2d_us": round(timed(other) * 1e3, 1), "conv2d_kernel": other_name,
+                   "auto_us": round(timed(auto) * 1e3, 1), "auto_takes": {1: "registers", 2: "dma", 3: "gemm"}[builtin_loader(auto.args)],
+                   "vendor_us": round(timed(lambda: torch.nn.functional.conv2d(x, w, bias)) * 1e3, 1)}
+            row["gbs_auto"] = round(2.0 * (x.numel() + w.numel() + y.numel()) / row["auto_us"] / 1e3, 1)
+            rows.append(row)
+    return rows
+
+
+def builtin_loader(conv_args):
+    """The loader `tnx_conv2d_default_config` names for this problem (tnx_conv_loader)."""
+    import ctypes
+
+    from tritonix_amd import _C
+
+    probe = type(conv_args).from_buffer_copy(conv_args)
+    st = _C.load().tnx_conv2d_default_config(ctypes.byref(probe))
+    assert st == _C.OK, _C.strerror(st)
+    return probe.loader
+
+
 def mfma_ceiling(torch, dev, dtype_code, peak):
     """T(FL)OP/s of the MFMA-only loop: {"16x16": {"random": .., "zeros": ..}, "32x32": {...}} (same protocol as the
     kernels: pre-roll, then one HIP-event pair around back-to-back launches on the launch stream)."""
@@ -315,6 +377,8 @@ def main():
                                "i8": mfma_ceiling(torch, dev, _C.I8, PEAK["i8"])}
     if args.shape_sweep:
         out["shape_sweep"] = shape_sweep(torch, dev, mm)
+    if args.conv1x1_sweep:
+        out["conv1x1_sweep"] = conv1x1_sweep(torch, dev)
     extras_wanted = [s for s in only if s != "C2"]
     if extras_wanted:
         out["per_config"] = extras(torch, dev, oracle, mm, sg, args, operands, extras_wanted)
@@ -412,7 +476,7 @@ def headline(torch, dev, oracle, mm, args, operands, out):
 
 
 def default_loader(conv_args):
-    """Which of the two conv2d kernels a launch with these arguments runs (tnx_conv_loader), by asking the library."""
+    """Which of the conv2d kernels a launch with these arguments runs (tnx_conv_loader), by asking the library."""
     import ctypes
 
     from tritonix_amd import _C
@@ -586,7 +650,7 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
                                                     gm, gn, gk, **cfg)
             r = measure(name, lambda i: lc(), flops, bytes_, "bf16", "mfma")
             r["tile"] = cfg
-            r["loader"] = {1: "registers", 2: "dma"}[default_loader(lc.args)]
+            r["loader"] = {1: "registers", 2: "dma", 3: "gemm"}[default_loader(lc.args)]
             r["workload"] = (f"conv2d forward bf16: input [{n_},{c_},{hw_},{hw_}], weight [{k_},{c_},{f_},{f_}], bias, "
                              f"stride {st_}, padding {pd_}")
             ref = oracle.reference_conv2d(x_cpu[5:6], w_cpu, b_cpu, *geo)

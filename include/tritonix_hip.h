@@ -236,11 +236,18 @@ typedef struct tnx_conv2d_args {
  * aligned weight; tiles of 128 or 256 channels x 128 or 256 pixels).  With TNX_CONV_LOADER_AUTO and no tile given
  * the library takes the direct-to-LDS kernel whenever the problem allows it and has enough tiles to fill the chip;
  * with a tile given it takes it when the tile exists only there, or exists in both and the problem allows it.
+ * A third way serves 1x1 filters with unit stride and no padding: such a layer is, image by image, the plain GEMM
+ * out[n] = weight[c_out, c_in] x input[n][c_in, h * w] (+ bias per row), and TNX_CONV_LOADER_GEMM runs it on the
+ * GEMM tile kernels themselves, all images in one grid (tile = block_cout x block_pixels x block_k of any built GEMM
+ * tile up to 128x128, or all three zero for a built-in choice; any c_in, any h * w).  TNX_CONV_LOADER_AUTO takes it only with the
+ * built-in tile, and there where it was measured ahead: wherever the direct-to-LDS kernel is not available, and on
+ * images of 2048 pixels or more whose rows are whole 16-byte units.
  * Asking for a loader the problem or tile does not allow returns TNX_E_UNSUPPORTED. */
 enum tnx_conv_loader {
   TNX_CONV_LOADER_AUTO = 0,
   TNX_CONV_LOADER_REGISTERS = 1,
-  TNX_CONV_LOADER_DMA = 2
+  TNX_CONV_LOADER_DMA = 2,
+  TNX_CONV_LOADER_GEMM = 3
 };
 
 /* Launch one conv2d forward.  Returns a tnx_status.  Asynchronous, allocates nothing. */

@@ -56,20 +56,33 @@ def test_default_config_names_a_built_tile():
     lib = _C.load()
     built = set(_C.conv2d_kernel_names())
     assert len(built) >= 16
-    loaders = {_C.CONV_LOADER_REGISTERS: "registers", _C.CONV_LOADER_DMA: "dma"}
+    gemm_tiles = {tuple(name.split()[:4]) for name in _C.kernel_names()}
+    loaders = {_C.CONV_LOADER_REGISTERS: "registers", _C.CONV_LOADER_DMA: "dma", _C.CONV_LOADER_GEMM: "gemm"}
+    one_by_one = dict(filter_h=1, filter_w=1, pad_h=0, pad_w=0)
     seen = set()
-    for kw in (dict(), dict(c_out=512, c_in=512, batch=32), dict(c_out=8, c_in=3, filter_h=1, filter_w=1, pad_h=0, pad_w=0),
+    for kw in (dict(), dict(c_out=512, c_in=512, batch=32), dict(c_out=8, c_in=3, **one_by_one),
                dict(batch=1, h_in=4, w_in=4), dict(c_in=64, c_out=256, h_in=56, w_in=56, batch=32),
-               dict(c_in=64, c_out=128, h_in=28, w_in=28, batch=8), dict(c_in=64, c_out=128, stride_w=2)):
+               dict(c_in=64, c_out=128, h_in=28, w_in=28, batch=8), dict(c_in=64, c_out=128, stride_w=2),
+               dict(c_in=64, c_out=256, h_in=56, w_in=56, batch=32, **one_by_one),
+               dict(c_in=1024, c_out=256, h_in=14, w_in=14, batch=32, **one_by_one),
+               dict(c_in=100, c_out=256, h_in=14, w_in=14, batch=32, **one_by_one)):
         a = _args(**kw)
         assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK
-        assert f"bf16 {a.block_cout} {a.block_pixels} {a.block_k} {loaders[a.loader]}" in built
+        if a.loader == _C.CONV_LOADER_GEMM:
+            assert ("bf16", str(a.block_cout), str(a.block_pixels), str(a.block_k)) in gemm_tiles
+        else:
+            assert f"bf16 {a.block_cout} {a.block_pixels} {a.block_k} {loaders[a.loader]}" in built
         assert a.group_pixels == 8
         assert lib.tnx_conv2d_supported(ctypes.byref(a)) == _C.OK
         seen.add((a.block_cout, a.block_pixels, loaders[a.loader]))
     # c_in * 9 a multiple of 64 and unit stride along w: the direct-to-LDS kernel; 256 channels wide when that leaves
     # two tiles per CU
     assert (256, 128, "dma") in seen and (128, 128, "dma") in seen and (128, 64, "registers") in seen
+    # 1x1 layers: the GEMM route on 56x56 images and wherever the direct-to-LDS kernel does not apply (c_in = 3, 100),
+    # the direct-to-LDS kernel on a 14x14 image with c_in a multiple of 64
+    assert (128, 128, "gemm") in seen and (64, 64, "gemm") in seen
+    a = _args(c_in=1024, c_out=256, h_in=14, w_in=14, batch=32, **one_by_one)
+    assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK and a.loader == _C.CONV_LOADER_DMA
 
 
 def test_loader_requests():
@@ -77,7 +90,8 @@ def test_loader_requests():
     ok = dict(c_in=64, c_out=128, block_pixels=128, block_cout=128, block_k=64)
     assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_DMA, **ok))) == _C.OK
     assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_REGISTERS, **ok))) == _C.OK
-    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=3, **ok))) == _C.E_INVALID
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=4, **ok))) == _C.E_INVALID
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=-1, **ok))) == _C.E_INVALID
     # stride along w, or c_in * R * S not a multiple of 64: only the register-staged kernel
     for bad in (dict(stride_w=2), dict(c_in=16)):
         kw = dict(ok, **bad)
@@ -86,6 +100,28 @@ def test_loader_requests():
     # a tile only one of the two kernels has
     assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_DMA, c_in=64, block_pixels=64, block_cout=64,
                                                        block_k=64))) == _C.E_UNSUPPORTED
+
+
+def test_gemm_route_requests():
+    """The GEMM route serves 1x1 filters with unit stride and no padding, on any built GEMM tile or its own choice."""
+    lib = _C.load()
+    flat = dict(filter_h=1, filter_w=1, pad_h=0, pad_w=0, loader=_C.CONV_LOADER_GEMM)
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(**flat))) == _C.OK
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(c_in=7, h_in=5, w_in=3, c_out=5, **flat))) == _C.OK
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(block_cout=128, block_pixels=128, block_k=64, **flat))) == _C.OK
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(block_cout=64, block_pixels=128, block_k=32, **flat))) == _C.OK
+    # the 256-wide GEMM tiles carry no problem index and no bias
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(block_cout=256, block_pixels=256, block_k=64, **flat))) == _C.E_UNSUPPORTED
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(dil_h=3, dil_w=2, **flat))) == _C.OK     # one tap: dilation has no effect
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(block_cout=96, block_pixels=128, block_k=64, **flat))) == _C.E_UNSUPPORTED
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(block_cout=128, block_pixels=0, block_k=64, **flat))) == _C.E_UNSUPPORTED
+    for bad in (dict(filter_h=3, pad_h=1), dict(stride_h=2), dict(stride_w=2), dict(pad_w=1)):
+        assert lib.tnx_conv2d_supported(ctypes.byref(_args(**dict(flat, **bad)))) == _C.E_UNSUPPORTED
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_GEMM))) == _C.E_UNSUPPORTED   # the 3x3 default
+    # a caller's tile with "auto" names a conv2d kernel, never the GEMM route: a tile only the GEMM kernels have is refused
+    only_gemm = dict(block_cout=32, block_pixels=64, block_k=64, c_in=64, filter_h=1, filter_w=1, pad_h=0, pad_w=0)
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(**only_gemm))) == _C.E_UNSUPPORTED
+    assert lib.tnx_conv2d_supported(ctypes.byref(_args(loader=_C.CONV_LOADER_GEMM, **only_gemm))) == _C.OK
 
 
 def test_every_reference_candidate_is_built():

@@ -132,6 +132,73 @@ def test_seeded_random_geometries_on_both_kernels(device):
         assert torch.equal(dma, regs), what
 
 
+# 1x1 filters, unit stride, no padding: n, c_in, h, w, c_out, bias dtype (None: no bias)
+GEMM_ROUTE_CASES = [
+    (2, 64, 16, 16, 128, torch.float32),       # rows of 512 bytes, K one slab
+    (3, 100, 13, 7, 70, "same"),               # ragged everywhere: c_in, plane of 91 pixels, channels
+    (2, 256, 56, 56, 64, "same"),              # the large-image layer "auto" hands to this route
+    (4, 2048, 7, 7, 512, None),                # long K, plane of 49 pixels (rows of 98 bytes)
+    (33, 24, 5, 5, 40, "same"),                # many small images
+    (1, 7, 3, 1, 5, torch.float32),            # smaller than one tile in every direction
+    (2, 192, 14, 14, 1000, "same"),            # channels ragged against 64 and 128
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_route_for_1x1_layers(dtype, device):
+    """A 1x1 layer is the GEMM out[n] = W x X[n] image by image; the GEMM route runs it on the GEMM tile kernels, all
+    images in one grid, bias added to the fp32 sum.  Against the oracle on the library's own tile and on named tiles;
+    with a 64-deep K slab it adds the same products in the same order as the conv2d kernels, so it must also agree
+    with the register-staged kernel bit for bit."""
+    for i, (n, c, h, w, k, bias) in enumerate(GEMM_ROUTE_CASES):
+        g = torch.Generator().manual_seed(100 + i)
+        x = torch.randn(n, c, h, w, generator=g).to(dtype)
+        wt = (torch.randn(k, c, 1, 1, generator=g) / c ** 0.5).to(dtype)
+        b = None if bias is None else torch.randn(k, generator=g).to(dtype if bias == "same" else bias)
+        geo = ((1, 1), (0, 0), (1, 1))
+        ref = oracle.reference_conv2d(x, wt, b, *geo)
+        xd, wd, bd = x.to(device), wt.to(device), None if b is None else b.to(device)
+        regs = conv2d_forward(xd, wd, bd, *geo, config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64, LOADER="registers"))
+        assert oracle.within_tolerance(regs, ref)[0], (i, dtype)
+        for (bm, bn, bk) in [(0, 0, 0), (64, 64, 64), (128, 128, 64), (128, 64, 64), (64, 32, 64), (128, 128, 32)]:
+            cfg = dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, LOADER="gemm")
+            canvas = torch.full((n * k * h * w + 64,), float("nan"), dtype=dtype, device=device)
+            out = canvas[32:32 + n * k * h * w].view(n, k, h, w)
+            conv2d_forward_kernel[(1,)](out, xd, wd, bd, n, c, h, w, k, h, w, 1, 1, 1, 1, 0, 0, 1, 1, n * h * w, k, c,
+                                        GROUP_SIZE_M=8, **cfg)
+            ok, err, rel = oracle.within_tolerance(out, ref)
+            assert ok, (i, dtype, cfg, err, rel)
+            assert bool(torch.isnan(canvas[:32]).all()) and bool(torch.isnan(canvas[32 + n * k * h * w:]).all()), (i, dtype, cfg)
+            if bk == 64 or bk == 0:
+                assert torch.equal(out, regs), (i, dtype, cfg)
+
+
+def test_gemm_route_follows_dilation_free_geometry_only(device):
+    """Dilation has no effect on a single tap; stride or padding take the layer off the GEMM route."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 64, 12, 12, generator=g).bfloat16().to(device)
+    wt = (torch.randn(96, 64, 1, 1, generator=g) / 8).bfloat16().to(device)
+    cfg = dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0, LOADER="gemm")
+    plain = conv2d_forward(x, wt, None, (1, 1), (0, 0), (1, 1), config=cfg)
+    assert torch.equal(conv2d_forward(x, wt, None, (1, 1), (0, 0), (3, 2), config=cfg), plain)
+    for stride, padding in (((2, 1), (0, 0)), ((1, 1), (0, 1))):
+        with pytest.raises(ValueError):
+            conv2d_forward(x, wt, None, stride, padding, (1, 1), config=cfg)
+
+
+def test_tuner_times_the_gemm_route_on_1x1_layers(device):
+    conv._CONV_FWD_CONFIG_CACHE.clear()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(8, 256, 56, 56, generator=g).bfloat16()
+    wt = (torch.randn(64, 256, 1, 1, generator=g) / 16).bfloat16()
+    out = conv2d_forward(x.to(device), wt.to(device))
+    assert oracle.within_tolerance(out[:1], oracle.reference_conv2d(x[:1], wt, None, (1, 1), (0, 0), (1, 1)))[0]
+    (cfg,) = conv._CONV_FWD_CONFIG_CACHE.values()
+    assert cfg.get("LOADER", "auto") in ("auto", "gemm")
+    again = conv2d_forward(x.to(device), wt.to(device))
+    assert torch.equal(out, again)
+
+
 def test_loader_that_does_not_fit_is_refused(device):
     x, wt, b, stride, padding, dilation = _inputs(CASES["1x1_stride2"], torch.bfloat16)
     with pytest.raises(ValueError):           # stride_w == 2

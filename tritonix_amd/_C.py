@@ -28,7 +28,7 @@ STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
 # enum tnx_lds_op
 LDS_READ_B128, LDS_WRITE_B128, LDS_READ_TR16_B64, LDS_READ_TR8_B64 = 0, 1, 2, 3
 # enum tnx_conv_loader
-CONV_LOADER_AUTO, CONV_LOADER_REGISTERS, CONV_LOADER_DMA = 0, 1, 2
+CONV_LOADER_AUTO, CONV_LOADER_REGISTERS, CONV_LOADER_DMA, CONV_LOADER_GEMM = 0, 1, 2, 3
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
            "tnx_gemm_default_config", "tnx_tile_coords", "tnx_probe_mfma", "tnx_probe_lds", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",

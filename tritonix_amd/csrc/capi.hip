@@ -198,11 +198,35 @@ static int compute_units(int* out) {
 
 extern "C" int tnx_gemm_supported(const tnx_gemm_args* a) { return supported_impl(a, nullptr, nullptr, false); }
 
-extern "C" int tnx_gemm(const tnx_gemm_args* a) {
+extern "C" int tnx_gemm(const tnx_gemm_args* a) { return tnx::gemm_launch(a, nullptr); }
+
+bool tnx::gemm_tile_for(int dtype, int bm, int bn, int bk, int* num_warps, int* num_stages) {
+  int ng = 0;
+  const KernelGroup* g = tnx_kernel_groups(&ng);
+  const KernelEntry* best = nullptr;
+  for (int i = 0; i < ng; ++i)
+    for (int j = 0; j < g[i].count; ++j) {
+      const KernelEntry& e = g[i].entries[j];
+      if (e.dtype != dtype || e.bm != bm || e.bn != bn || e.bk != bk || !e.fast || e.bm * e.bn > 128 * 128) continue;
+      // four waves; three ring slots (these layers stream their operands once: a second workgroup on the CU is worth
+      // more than a deeper ring), else the deepest ring
+      auto score = [](const KernelEntry& k) { return (k.nw == 4 ? 100 : 0) + (k.stages == 3 ? 50 : 0) + k.stages; };
+      if (!best || score(e) > score(*best)) best = &e;
+    }
+  if (!best) return false;
+  *num_warps = best->nw;
+  *num_stages = best->stages;
+  return true;
+}
+
+int tnx::gemm_launch(const tnx_gemm_args* a, const GemmBatch* extra) {
   const KernelEntry* e = nullptr;
   bool fast = false, bt = false, tail_slab = false;
   int st = supported_impl(a, &e, &fast, true, &bt, &tail_slab);
   if (st != TNX_OK) return st;
+  if (extra && (e->bm * e->bn > 128 * 128 || a->split_k != 1 || (a->schedule & TNX_SCHED_PERSISTENT) || is_skinny_cfg(a) || extra->batch < 1 ||
+                a->epilogue != TNX_EPI_NONE || (extra->bias && a->in_dtype == TNX_I8)))
+    return TNX_E_UNSUPPORTED;
   if (!a->a || !a->b || !a->c) {
     if (a->m == 0 || a->n == 0) return TNX_OK;
     if (!a->c || (a->k > 0 && (!a->a || !a->b))) return TNX_E_INVALID;
@@ -239,6 +263,16 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
   p.c_vec_ok = a->stride_cn == 1 && ((a->stride_cm * es_out) % 16) == 0 && (((uintptr_t)a->c) % 16) == 0;
   p.c_row_ok = a->stride_cn == 1;
   p.tail_slab = tail_slab ? 1 : 0;
+  int64_t problems = 1;
+  if (extra) {
+    p.batch = extra->batch;
+    p.b_batch_bytes = extra->b_batch_bytes;
+    p.c_batch_bytes = extra->c_batch_bytes;
+    p.cv.bias = (const uint8_t*)extra->bias;
+    p.cv.bias_dtype = extra->bias_dtype;
+    problems = extra->batch;
+    if ((int64_t)p.tiles_m * p.tiles_n * problems > 0x7fffffffll) return TNX_E_UNSUPPORTED;
+  }
 
   hipStream_t stream = (hipStream_t)a->stream;
   hipError_t err;
@@ -251,7 +285,7 @@ extern "C" int tnx_gemm(const tnx_gemm_args* a) {
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     err = e->persist(p, (unsigned)(tiles < cus ? tiles : cus), stream);
   } else {
-    unsigned grid = a->split_k > 1 ? (unsigned)(p.split_tile0 + ncut * a->split_k) : (unsigned)(p.tiles_m * p.tiles_n);
+    unsigned grid = a->split_k > 1 ? (unsigned)(p.split_tile0 + ncut * a->split_k) : (unsigned)((int64_t)p.tiles_m * p.tiles_n * problems);
     err = (bt ? e->fast_bt : fast ? e->fast : e->generic)(p, grid, stream);
   }
   if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }

@@ -162,20 +162,99 @@ static bool dma_problem_ok(const tnx_conv2d_args* a, int h_out, int w_out, bool 
 
 struct Resolved {
   const ConvEntry* reg;      // register-staged kernel, or
-  const KernelEntry* dma;    // the GEMM kernel's conv2d variant
+  const KernelEntry* dma;    // the GEMM kernel's conv2d variant, or
+  bool gemm;                 // the plain GEMM kernel, one problem per image (1x1 filters, unit stride, no padding)
+  int gemm_warps, gemm_stages;
   int bcout, bpix, bk;
   int h_out, w_out;
 };
+
+// A 1x1 filter with unit stride and no padding: out[n] = W[c_out, c_in] x X[n][c_in, h*w] + bias, image by image.
+static bool gemm_problem_ok(const tnx_conv2d_args* a) {
+  return a->filter_h == 1 && a->filter_w == 1 && a->stride_h == 1 && a->stride_w == 1 && a->pad_h == 0 && a->pad_w == 0;
+}
+
+// Built-in tile for that GEMM: 128 x 128, narrowed to 64 channels or 64 pixels where the layer is that small or the
+// grid would leave CUs idle; a short ring where K is short (measured on the 1x1 layers of a ResNet-50, batch 32:
+// 128x128 two stages on c_in 64..256, 64x128 and 64x64 on the 14x14 and 7x7 layers).
+static bool builtin_gemm_tile(const tnx_conv2d_args* a, int* bcout, int* bpix, int* bk, int* nw, int* st) {
+  const int64_t hw = (int64_t)a->h_in * a->w_in;
+  int bm = a->c_out <= 64 ? 64 : 128, bn = hw <= 64 ? 64 : 128;
+  auto tiles = [&](int m, int n) { return (((int64_t)a->c_out + m - 1) / m) * ((hw + n - 1) / n) * a->batch; };
+  if (tiles(bm, bn) < 256 && bm > 64) bm = 64;
+  if (tiles(bm, bn) < 256 && bn > 64) bn = 64;
+  *bcout = bm; *bpix = bn; *bk = 64;
+  if (!gemm_tile_for(a->dtype, bm, bn, 64, nw, st)) return false;
+  if (bm == 128 && bn == 128 && a->c_in <= 256) { *nw = 4; *st = 2; }   // two workgroups per CU instead of a deeper ring
+  return true;
+}
+
+static void fill_gemm(const tnx_conv2d_args* a, const Resolved& r, tnx_gemm_args* g, GemmBatch* x) {
+  const int64_t hw = (int64_t)a->h_in * a->w_in;
+  *g = tnx_gemm_args{};
+  g->a = a->weight; g->b = a->input; g->c = a->output;
+  g->m = a->c_out; g->n = hw; g->k = a->c_in;
+  g->stride_am = a->c_in; g->stride_ak = 1;
+  g->stride_bk = hw; g->stride_bn = 1;
+  g->stride_cm = hw; g->stride_cn = 1;
+  g->in_dtype = a->dtype; g->out_dtype = a->dtype;
+  g->block_m = r.bcout; g->block_n = r.bpix; g->block_k = r.bk;
+  g->group_m = 8; g->split_k = 1;
+  g->num_stages = r.gemm_stages; g->num_warps = r.gemm_warps;
+  g->epilogue = TNX_EPI_NONE;
+  g->stream = a->stream;
+  x->batch = a->batch;
+  x->b_batch_bytes = (int64_t)a->c_in * hw * 2;
+  x->c_batch_bytes = (int64_t)a->c_out * hw * 2;
+  x->bias = a->bias;
+  x->bias_dtype = a->bias_dtype;
+}
 
 static int resolve(const tnx_conv2d_args* a, Resolved* r, bool inspect_ptrs) {
   int32_t h_out = 0, w_out = 0;
   const int st = check_problem(a, &h_out, &w_out);
   if (st != TNX_OK) return st;
-  if (a->loader < TNX_CONV_LOADER_AUTO || a->loader > TNX_CONV_LOADER_DMA) return TNX_E_INVALID;
+  if (a->loader < TNX_CONV_LOADER_AUTO || a->loader > TNX_CONV_LOADER_GEMM) return TNX_E_INVALID;
   const int64_t pixels = (int64_t)a->batch * h_out * w_out;
   const bool dma_ok = dma_problem_ok(a, h_out, w_out, inspect_ptrs);
   int bcout = a->block_cout, bpix = a->block_pixels, bk = a->block_k;
   const bool builtin = bcout == 0 && bpix == 0 && bk == 0;
+  *r = Resolved{};
+  r->h_out = h_out; r->w_out = w_out;
+  if (a->loader == TNX_CONV_LOADER_GEMM && !gemm_problem_ok(a)) return TNX_E_UNSUPPORTED;
+  // "auto" takes the GEMM route only with the built-in tile (a caller's tile names a conv2d kernel), and there where it
+  // was measured ahead on 1x1 layers of a ResNet-50 at batch 8, 32 and 128: wherever the direct-to-LDS conv2d kernel is
+  // not available (1.1x to 5x over the register-staged one), and on large images with 16-byte rows (56x56: 1.0x to 1.4x).
+  // On 28x28 and smaller images the conv2d kernel packs the pixels of all images into its tiles, the GEMM route pads
+  // every image to whole tiles, and neither wins throughout (0.74x to 1.7x).
+  bool try_gemm = a->loader == TNX_CONV_LOADER_GEMM;
+  if (a->loader == TNX_CONV_LOADER_AUTO && builtin && gemm_problem_ok(a)) {
+    int t0 = 0, t1 = 0, t2 = 0;
+    const int64_t hw = (int64_t)a->h_in * a->w_in;
+    try_gemm = !(dma_ok && builtin_dma_tile(a, h_out, w_out, &t0, &t1, &t2)) || (hw >= 2048 && hw % 8 == 0);
+  }
+  if (try_gemm) {
+    int nw = 0, st2 = 0;
+    bool found = false;
+    if (builtin) found = builtin_gemm_tile(a, &bcout, &bpix, &bk, &nw, &st2);
+    else if (bcout > 0 && bpix > 0 && bk > 0) found = gemm_tile_for(a->dtype, bcout, bpix, bk, &nw, &st2);
+    if (found) {
+      r->gemm = true; r->gemm_warps = nw; r->gemm_stages = st2;
+      r->bcout = bcout; r->bpix = bpix; r->bk = bk;
+      tnx_gemm_args g;
+      GemmBatch x;
+      fill_gemm(a, *r, &g, &x);
+      if (!inspect_ptrs) { g.a = nullptr; g.b = nullptr; g.c = nullptr; }
+      const int sg = tnx_gemm_supported(&g);
+      if (sg == TNX_OK && ((int64_t)((a->c_out + bcout - 1) / bcout) * (((int64_t)a->h_in * a->w_in + bpix - 1) / bpix) * a->batch < (1ll << 31)))
+        return TNX_OK;
+      if (a->loader == TNX_CONV_LOADER_GEMM) return sg == TNX_OK ? TNX_E_UNSUPPORTED : sg;
+      r->gemm = false;
+    } else if (a->loader == TNX_CONV_LOADER_GEMM) {
+      return TNX_E_UNSUPPORTED;
+    }
+    bcout = a->block_cout; bpix = a->block_pixels; bk = a->block_k;
+  }
   bool want_dma = a->loader == TNX_CONV_LOADER_DMA;
   if (builtin) {
     if (a->loader != TNX_CONV_LOADER_REGISTERS && dma_ok && builtin_dma_tile(a, h_out, w_out, &bcout, &bpix, &bk)) want_dma = true;
@@ -292,7 +371,7 @@ extern "C" int tnx_conv2d_default_config(tnx_conv2d_args* a) {
   a->block_pixels = r.bpix;
   a->block_k = r.bk;
   a->group_pixels = 8;
-  a->loader = r.dma ? TNX_CONV_LOADER_DMA : TNX_CONV_LOADER_REGISTERS;
+  a->loader = r.gemm ? TNX_CONV_LOADER_GEMM : r.dma ? TNX_CONV_LOADER_DMA : TNX_CONV_LOADER_REGISTERS;
   return TNX_OK;
 }
 
@@ -306,6 +385,12 @@ extern "C" int tnx_conv2d_forward(const tnx_conv2d_args* a) {
   if (a->bias && ((uintptr_t)a->bias & (a->bias_dtype == TNX_F32 ? 3 : 1))) return TNX_E_INVALID;
   unsigned grid = 0;
   hipError_t err;
+  if (r.gemm) {
+    tnx_gemm_args g;
+    GemmBatch x;
+    fill_gemm(a, r, &g, &x);
+    return gemm_launch(&g, &x);
+  }
   if (r.dma) {
     GemmParams p;
     fill_dma(a, r, &p, &grid);

@@ -5,6 +5,8 @@
 
 #include "gemm_tile.h"
 
+struct tnx_gemm_args;
+
 namespace tnx {
 
 typedef hipError_t (*launch_fn)(const GemmParams& p, unsigned grid, hipStream_t stream);
@@ -21,6 +23,20 @@ struct KernelEntry {
 
 // records the hipError_t behind a TNX_E_HIP for tnx_last_hip_error() (per thread)
 void note_hip_error(int err);
+// tnx_gemm with `batch` problems in one grid -- same A, problem i reads b + i * b_batch_bytes and writes
+// c + i * c_batch_bytes -- and an optional bias per row of C, added to the fp32 sum before the rounding (float types).
+// Uncut, non-persistent launches of tiles up to 128x128 only (multi_problem_tile).  conv2d's 1x1 layers are this GEMM,
+// one problem per image.
+struct GemmBatch {
+  int batch;
+  int64_t b_batch_bytes, c_batch_bytes;
+  const void* bias;
+  int bias_dtype;
+};
+int gemm_launch(const tnx_gemm_args* a, const GemmBatch* extra);
+// waves and stages of a built tile with these dimensions that gemm_launch takes with a GemmBatch (four waves and
+// three ring slots first); false: none built
+bool gemm_tile_for(int dtype, int bm, int bn, int bk, int* num_warps, int* num_stages);
 
 struct KernelGroup {
   KernelEntry* entries;

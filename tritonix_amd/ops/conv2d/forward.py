@@ -39,7 +39,8 @@ _CANDIDATE_CONFIGS = [
 ]
 _CONV_FWD_CONFIG_CACHE: Dict[tuple, dict] = {}
 # optional launch keyword LOADER (no counterpart in the reference): which of the two kernels moves the slabs
-_LOADERS = {"auto": _C.CONV_LOADER_AUTO, "registers": _C.CONV_LOADER_REGISTERS, "dma": _C.CONV_LOADER_DMA}
+_LOADERS = {"auto": _C.CONV_LOADER_AUTO, "registers": _C.CONV_LOADER_REGISTERS, "dma": _C.CONV_LOADER_DMA,
+            "gemm": _C.CONV_LOADER_GEMM}
 
 
 def output_size(h_in: int, w_in: int, filter_h: int, filter_w: int, stride, padding, dilation) -> Tuple[int, int]:
@@ -215,7 +216,8 @@ def conv2d_forward(
     """conv2d forward on the HIP kernel; same arguments and result as tritonix/ops/conv2d/forward.py:202-311.
 
     ``config=None`` times the candidate tiles once per problem key and remembers the fastest, as the reference
-    does; ``config={"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K"[, "GROUP_SIZE_M"]}`` launches that tile.
+    does; ``config={"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K"[, "GROUP_SIZE_M"][, "LOADER"]}`` launches that tile
+    (all three sizes 0: the library's own choice; ``LOADER`` is "auto", "registers", "dma" or "gemm").
     Returns a new [N, C_OUT, H_OUT, W_OUT] tensor of the input's dtype."""
     assert input.is_contiguous(), "Input must be contiguous NCHW"
     assert weight.is_contiguous(), "Weight must be contiguous KCRS"
@@ -231,7 +233,7 @@ def conv2d_forward(
     out = input.new_empty((n, c_out, h_out, w_out))
 
     def launch(bm, bn, bk, g, loader="auto", dst=out):
-        conv2d_forward_kernel[(cdiv(gemm_m, bm), cdiv(gemm_n, bn))](
+        conv2d_forward_kernel[(cdiv(gemm_m, bm or 1), cdiv(gemm_n, bn or 1))](
             dst, input, weight, bias, n, c_in, h_in, w_in, c_out, h_out, w_out, r, s,
             stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], gemm_m, gemm_n, gemm_k,
             BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=g, USE_TF32=use_tf32, LOADER=loader)
@@ -248,6 +250,14 @@ def conv2d_forward(
                     continue
                 if t < best_time:
                     best_time, best = t, dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=g)
+            if (r, s) == (1, 1) and stride == (1, 1) and padding == (0, 0):
+                # a 1x1 layer is a plain GEMM per image: the library's GEMM route with its own tile is one more candidate
+                try:
+                    t = _time_kernel(lambda: launch(0, 0, 0, 8, "gemm"))
+                    if t < best_time:
+                        best_time, best = t, dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0, GROUP_SIZE_M=8, LOADER="gemm")
+                except (ValueError, _C.OutOfResources):
+                    pass
             if best is None:
                 raise RuntimeError("conv2d_forward: no candidate tile could be launched")
             _CONV_FWD_CONFIG_CACHE[key] = cfg = best
