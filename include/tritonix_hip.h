@@ -239,9 +239,8 @@ typedef struct tnx_conv2d_args {
  * A third way serves 1x1 filters with unit stride and no padding: such a layer is, image by image, the plain GEMM
  * out[n] = weight[c_out, c_in] x input[n][c_in, h * w] (+ bias per row), and TNX_CONV_LOADER_GEMM runs it on the
  * GEMM tile kernels themselves, all images in one grid (tile = block_cout x block_pixels x block_k of any built GEMM
- * tile up to 128x128, or all three zero for a built-in choice; any c_in, any h * w).  TNX_CONV_LOADER_AUTO takes it only with the
- * built-in tile, and there where it was measured ahead: wherever the direct-to-LDS kernel is not available, and on
- * images of 2048 pixels or more whose rows are whole 16-byte units.
+ * tile up to 128x128, or all three zero for a built-in choice; any c_in, any h * w).  TNX_CONV_LOADER_AUTO takes it with the
+ * built-in tile on every such layer (a tile given by the caller names a conv2d kernel).
  * Asking for a loader the problem or tile does not allow returns TNX_E_UNSUPPORTED. */
 enum tnx_conv_loader {
   TNX_CONV_LOADER_AUTO = 0,

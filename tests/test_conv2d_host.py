@@ -78,11 +78,13 @@ def test_default_config_names_a_built_tile():
     # c_in * 9 a multiple of 64 and unit stride along w: the direct-to-LDS kernel; 256 channels wide when that leaves
     # two tiles per CU
     assert (256, 128, "dma") in seen and (128, 128, "dma") in seen and (128, 64, "registers") in seen
-    # 1x1 layers: the GEMM route on 56x56 images and wherever the direct-to-LDS kernel does not apply (c_in = 3, 100),
-    # the direct-to-LDS kernel on a 14x14 image with c_in a multiple of 64
+    # 1x1 layers with unit stride and no padding: the GEMM route
     assert (128, 128, "gemm") in seen and (64, 64, "gemm") in seen
-    a = _args(c_in=1024, c_out=256, h_in=14, w_in=14, batch=32, **one_by_one)
-    assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK and a.loader == _C.CONV_LOADER_DMA
+    for kw in (dict(c_in=1024, c_out=256, h_in=14, w_in=14, batch=32), dict(c_in=3, c_out=8), dict(c_in=64, c_out=64, h_in=7, w_in=7)):
+        a = _args(**kw, **one_by_one)
+        assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK and a.loader == _C.CONV_LOADER_GEMM
+    a = _args(c_in=64, c_out=64, stride_h=2, **one_by_one)
+    assert lib.tnx_conv2d_default_config(ctypes.byref(a)) == _C.OK and a.loader != _C.CONV_LOADER_GEMM
 
 
 def test_loader_requests():

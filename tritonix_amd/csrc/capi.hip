@@ -208,9 +208,16 @@ bool tnx::gemm_tile_for(int dtype, int bm, int bn, int bk, int* num_warps, int* 
     for (int j = 0; j < g[i].count; ++j) {
       const KernelEntry& e = g[i].entries[j];
       if (e.dtype != dtype || e.bm != bm || e.bn != bn || e.bk != bk || !e.fast || e.bm * e.bn > 128 * 128) continue;
-      // four waves; three ring slots (these layers stream their operands once: a second workgroup on the CU is worth
-      // more than a deeper ring), else the deepest ring
-      auto score = [](const KernelEntry& k) { return (k.nw == 4 ? 100 : 0) + (k.stages == 3 ? 50 : 0) + k.stages; };
+      // Eight waves and two ring slots first, then the shallowest ring: these problems stream their operands once
+      // through a short K loop, and what hides the latency of a tile's first slab and of its stores is more waves and a
+      // second workgroup on the CU, not a deeper ring (measured on GEMMs shaped like the 1x1 layers of a ResNet-50:
+      // 128x128x64 with 8 waves / 2 slots 39 us, 4 / 2 43 us, 4 / 3 75 us on [512 x 256] x [256 x 100352])
+      // A 64x64 tile is too little work for eight waves: four waves and three slots there (measured on the small
+      // layers, 2048 -> 512 channels at 7x7: 16.3 against 21.9 us).
+      auto score = [](const KernelEntry& k) {
+        const bool small = k.bm * k.bn <= 64 * 64;
+        return (k.nw == (small ? 4 : 8) ? 100 : 0) + (k.stages == (small ? 3 : 2) ? 50 : 0) - k.stages;
+      };
       if (!best || score(e) > score(*best)) best = &e;
     }
   if (!best) return false;

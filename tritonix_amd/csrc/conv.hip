@@ -175,8 +175,7 @@ static bool gemm_problem_ok(const tnx_conv2d_args* a) {
 }
 
 // Built-in tile for that GEMM: 128 x 128, narrowed to 64 channels or 64 pixels where the layer is that small or the
-// grid would leave CUs idle; a short ring where K is short (measured on the 1x1 layers of a ResNet-50, batch 32:
-// 128x128 two stages on c_in 64..256, 64x128 and 64x64 on the 14x14 and 7x7 layers).
+// grid would leave CUs idle (measured on the 1x1 layers of a ResNet-50 at batch 8, 32 and 128).
 static bool builtin_gemm_tile(const tnx_conv2d_args* a, int* bcout, int* bpix, int* bk, int* nw, int* st) {
   const int64_t hw = (int64_t)a->h_in * a->w_in;
   int bm = a->c_out <= 64 ? 64 : 128, bn = hw <= 64 ? 64 : 128;
@@ -184,9 +183,7 @@ static bool builtin_gemm_tile(const tnx_conv2d_args* a, int* bcout, int* bpix, i
   if (tiles(bm, bn) < 256 && bm > 64) bm = 64;
   if (tiles(bm, bn) < 256 && bn > 64) bn = 64;
   *bcout = bm; *bpix = bn; *bk = 64;
-  if (!gemm_tile_for(a->dtype, bm, bn, 64, nw, st)) return false;
-  if (bm == 128 && bn == 128 && a->c_in <= 256) { *nw = 4; *st = 2; }   // two workgroups per CU instead of a deeper ring
-  return true;
+  return gemm_tile_for(a->dtype, bm, bn, 64, nw, st);
 }
 
 static void fill_gemm(const tnx_conv2d_args* a, const Resolved& r, tnx_gemm_args* g, GemmBatch* x) {
@@ -222,17 +219,11 @@ static int resolve(const tnx_conv2d_args* a, Resolved* r, bool inspect_ptrs) {
   *r = Resolved{};
   r->h_out = h_out; r->w_out = w_out;
   if (a->loader == TNX_CONV_LOADER_GEMM && !gemm_problem_ok(a)) return TNX_E_UNSUPPORTED;
-  // "auto" takes the GEMM route only with the built-in tile (a caller's tile names a conv2d kernel), and there where it
-  // was measured ahead on 1x1 layers of a ResNet-50 at batch 8, 32 and 128: wherever the direct-to-LDS conv2d kernel is
-  // not available (1.1x to 5x over the register-staged one), and on large images with 16-byte rows (56x56: 1.0x to 1.4x).
-  // On 28x28 and smaller images the conv2d kernel packs the pixels of all images into its tiles, the GEMM route pads
-  // every image to whole tiles, and neither wins throughout (0.74x to 1.7x).
-  bool try_gemm = a->loader == TNX_CONV_LOADER_GEMM;
-  if (a->loader == TNX_CONV_LOADER_AUTO && builtin && gemm_problem_ok(a)) {
-    int t0 = 0, t1 = 0, t2 = 0;
-    const int64_t hw = (int64_t)a->h_in * a->w_in;
-    try_gemm = !(dma_ok && builtin_dma_tile(a, h_out, w_out, &t0, &t1, &t2)) || (hw >= 2048 && hw % 8 == 0);
-  }
+  // "auto" takes the GEMM route with the built-in tile (a caller's tile names a conv2d kernel) on every layer that is
+  // such a GEMM: measured on the 1x1 layers of a ResNet-50 at batch 8, 32 and 128 it is level with or ahead of the
+  // conv2d kernels on 34 of 36 (1.0x to 5.4x; 0.90x and 0.93x on 14x14 planes at batch 128, where it pads every image
+  // to whole pixel tiles and the conv2d kernel packs the pixels of all images).
+  const bool try_gemm = a->loader == TNX_CONV_LOADER_GEMM || (a->loader == TNX_CONV_LOADER_AUTO && builtin && gemm_problem_ok(a));
   if (try_gemm) {
     int nw = 0, st2 = 0;
     bool found = false;

@@ -540,6 +540,20 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
   static_assert(WCOLS % PK::OUTV == 0, "wave tile too narrow for 16-byte stores");
   raw* cp = (raw*)cbase;
   const uint32_t wbase0 = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
+  // A bias per row of C (conv2d's 1x1 layers): lane l fetches the values of rows l, l + 64, .. of the wave tile now,
+  // so that the loads fly under the first pass through the strip; the row loop below picks its value from the lane that holds it.
+  constexpr bool WITH_BIAS = BIAS && std::is_same<acc_s, float>::value && !GLU;
+  constexpr int NBR = (C::WTM + 63) / 64;
+  float bias_rows[NBR] = {};
+  if constexpr (WITH_BIAS) {
+    if (bias) {
+#pragma unroll
+      for (int r = 0; r < NBR; ++r) {
+        const int64_t g = gm0 + r * 64 + lane;
+        if (r * 64 + lane < C::WTM && g < m) bias_rows[r] = bias_value(bias, (int)g, bias_dtype);
+      }
+    }
+  }
 #pragma unroll
   for (int i0 = 0; i0 < C::TM; i0 += RB) {
     if (gm0 + i0 * MI >= m) break;                      // row-blocks past the last row hold nothing
@@ -574,12 +588,22 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
     for (int it0 = 0; it0 < ITERS; it0 += UNR) {
       // UNR rows of LDS reads are issued together, then converted and stored one after the other
       acc_s f[UNR][PK::NF];
+      float bv[UNR] = {};
 #pragma unroll
       for (int u = 0; u < UNR; ++u) {
         const int q = (it0 + u) * 64 + lane;
         int row = q / CPRW;
         const int cc = q % CPRW;
         if (ROWS * CPRW % 64 != 0 && row >= ROWS) row = ROWS - 1;
+        if constexpr (WITH_BIAS) {
+          const int rt = i0 * MI + row;                 // row of the wave tile: held by lane rt % 64 in bias_rows[rt / 64]
+          if (bias)
+#pragma unroll
+          for (int r = 0; r < NBR; ++r) {
+            const float t = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((rt & 63) * 4, __builtin_bit_cast(int, bias_rows[r])));
+            if ((rt >> 6) == r) bv[u] = t;
+          }
+        }
 #pragma unroll
         for (int x = 0; x < PK::NF / 4; ++x) {
           const i32x4 v = *TNX_LDS(i32x4, lds_strip + row * PITCH + (cc * PK::NF + 4 * x) * 4);
@@ -593,13 +617,11 @@ __device__ __forceinline__ void epilogue_store(ACC (&acc)[C::TM][C::TN], const S
         const int64_t gm = gm0 + i0 * MI + row;
         const int64_t gc = gc0 + cc * PK::OUTV;
         if ((ROWS * CPRW % 64 != 0 && row >= ROWS) || gm >= m) continue;
-        if constexpr (BIAS && std::is_same<acc_s, float>::value && !GLU) {
-          // a bias per row of C, added to the finished fp32 sum before the one rounding (conv2d's 1x1 layers)
-          if (bias) {
-            const float bv = bias_value(bias, (int)gm, bias_dtype);
+        if constexpr (WITH_BIAS) {
+          // added to the finished fp32 sum before the one rounding
+          if (bias)
 #pragma unroll
-            for (int x = 0; x < PK::NF; ++x) f[u][x] += bv;
-          }
+            for (int x = 0; x < PK::NF; ++x) f[u][x] += bv[u];
         }
         raw out[PK::OUTV];
         PK::run(f[u], epi, out);

@@ -34,8 +34,8 @@ struct GemmBatch {
   int bias_dtype;
 };
 int gemm_launch(const tnx_gemm_args* a, const GemmBatch* extra);
-// waves and stages of a built tile with these dimensions that gemm_launch takes with a GemmBatch (four waves and
-// three ring slots first); false: none built
+// waves and stages of a built tile with these dimensions that gemm_launch takes with a GemmBatch (eight waves and
+// two ring slots first); false: none built
 bool gemm_tile_for(int dtype, int bm, int bn, int bk, int* num_warps, int* num_stages);
 
 struct KernelGroup {
