@@ -160,7 +160,8 @@ def test_gemm_route_for_1x1_layers(dtype, device):
         xd, wd, bd = x.to(device), wt.to(device), None if b is None else b.to(device)
         regs = conv2d_forward(xd, wd, bd, *geo, config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64, LOADER="registers"))
         assert oracle.within_tolerance(regs, ref)[0], (i, dtype)
-        for (bm, bn, bk) in [(0, 0, 0), (64, 64, 64), (128, 128, 64), (128, 64, 64), (64, 32, 64), (128, 128, 32)]:
+        for (bm, bn, bk) in [(0, 0, 0), (64, 64, 64), (128, 128, 64), (128, 64, 64), (64, 32, 64), (128, 128, 32),
+                             (64, 256, 64), (64, 256, 32)]:    # the last: wave tiles of 128 rows, two bias values per lane
             cfg = dict(BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, LOADER="gemm")
             canvas = torch.full((n * k * h * w + 64,), float("nan"), dtype=dtype, device=device)
             out = canvas[32:32 + n * k * h * w].view(n, k, h, w)
