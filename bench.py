@@ -198,7 +198,8 @@ def sustain(step, seconds, flops):
 
 
 SWEEP_SHAPES = [(1, 4096, 4096), (8, 14336, 4096), (32, 4096, 14336), (64, 8192, 8192), (128, 8192, 8192),
-                (512, 4096, 4096), (1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096),
+                (512, 4096, 4096), (1024, 1024, 1024), (2048, 2048, 512), (2048, 2048, 2048), (1024, 4096, 4096),
+                (3072, 3072, 3072), (4096, 4096, 4096),
                 (4096, 4096, 4104), (4096, 4100, 4096), (4100, 4096, 4096)]
 
 
@@ -216,10 +217,10 @@ def shape_sweep(torch, dev, mm):
         kern = mm.gemm_splitk_kernel if cfg.get("split_k", 1) > 1 else mm.matmul_kernel
         c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
         ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), 1, n, 1, **cfg) for b in bs]
-        for i in range(20):
+        for i in range(200):     # the host spent the last seconds drawing random operands: bring the clocks back up
             ls[i % len(ls)]()
         ours = region_time(lambda i: ls[i % len(ls)](), 50)
-        for i in range(10):
+        for i in range(20):
             torch.matmul(a, bs[i % len(bs)], out=c)
         vendor = region_time(lambda i: torch.matmul(a, bs[i % len(bs)], out=c), 50)
         rows.append({"shape": [m, n, k], "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),

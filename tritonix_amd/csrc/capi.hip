@@ -429,6 +429,12 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     }
   }
   a->block_m = cand[bi][0]; a->block_n = cand[bi][1]; a->num_stages = cand[bi][2]; a->num_warps = cand[bi][3];
+  // The 128x128 tile, and the 64x128 tile of the 16-bit types, run with eight waves: problems that end up on them are
+  // a few rounds of short tiles, and two waves per SIMD hide more of a tile's start and end than one (measured on
+  // fifteen bf16 shapes from 768x3072x768 to 1024x4096x4096, three ring slots both: 1-14 % faster on every one, e.g.
+  // 2048^3 21.2 -> 19.6 us, 2048^2 x 512 9.4 -> 8.1 us, 1024^3 9.1 -> 7.9 us; int8 128x128 5-13 % on seven shapes,
+  // int8 64x128 mixed).
+  if (bi == 2 || (es == 2 && bi == 3)) a->num_warps = 8;
   // 16-bit problems with a short K loop (at most 64 slabs per tile) spend a visible share of every tile outside
   // it; two waves per SIMD cover that better than one (measured on 4096 x 28672 x 4096, gated: +2.4 %), at the
   // price of half again as many LDS reads, which is what loses on the long, power-limited 8192^3 loops.
