@@ -118,13 +118,24 @@ def cpu_time(fn, budget_s=8.0, max_reps=3):
     return sorted(ts)[len(ts) // 2], len(ts)
 
 
-def vendor_ms(fn, reps=20):
-    """Mean per-launch ms of a torch GPU op (the vendor BLAS), same event protocol as the kernels under test."""
+def pre_roll(fn):
+    """Untimed launches until the part is out of idle clocks: PRE_ROLL of them, repeated until 50 ms have passed (after
+    host-side work -- drawing operands, a CPU reference -- a short kernel would otherwise be timed at idle clocks)."""
     import torch
 
-    for i in range(PRE_ROLL):
-        fn(i)
-    torch.cuda.synchronize()
+    t0, i = time.perf_counter(), 0
+    while True:
+        for _ in range(PRE_ROLL):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 > 0.05:
+            return
+
+
+def vendor_ms(fn, reps=20):
+    """Mean per-launch ms of a torch GPU op (the vendor BLAS), same event protocol as the kernels under test."""
+    pre_roll(fn)
     return round(region_time(fn, 2 * reps), 4)
 
 
@@ -217,11 +228,9 @@ def shape_sweep(torch, dev, mm):
         kern = mm.gemm_splitk_kernel if cfg.get("split_k", 1) > 1 else mm.matmul_kernel
         c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
         ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), 1, n, 1, **cfg) for b in bs]
-        for i in range(200):     # the host spent the last seconds drawing random operands: bring the clocks back up
-            ls[i % len(ls)]()
+        pre_roll(lambda i: ls[i % len(ls)]())
         ours = region_time(lambda i: ls[i % len(ls)](), 50)
-        for i in range(20):
-            torch.matmul(a, bs[i % len(bs)], out=c)
+        pre_roll(lambda i: torch.matmul(a, bs[i % len(bs)], out=c))
         vendor = region_time(lambda i: torch.matmul(a, bs[i % len(bs)], out=c), 50)
         rows.append({"shape": [m, n, k], "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),
                      "gbs": round(2.0 * (m * k + k * n + m * n) / ours / 1e6, 1), "vendor_ms": round(vendor, 4),
@@ -258,16 +267,13 @@ def conv1x1_sweep(torch, dev):
                                                           1, 1, batch * hw * hw, c_out, c_in, LOADER=loader, **zero)
 
             def timed(fn):
-                for _ in range(20):
-                    fn()
+                pre_roll(lambda i: fn())
                 return region_time(lambda i: fn(), 50)
 
             other, other_name = bound("dma"), "dma"
             if _C.load().tnx_conv2d_supported(ctypes.byref(other.args)) != _C.OK:
                 other, other_name = bound("registers"), "registers"
             auto = bound("auto")
-            for _ in range(200):     # the host spent the last seconds drawing random tensors: bring the clocks back up
-                auto()
             row = {"batch": batch, "layer": [c_in, hw, c_out], "gemm_us": round(timed(bound("gemm")) * 1e3, 1),
                    "conv2d_us": round(timed(other) * 1e3, 1), "conv2d_kernel": other_name,
                    "auto_us": round(timed(auto) * 1e3, 1), "auto_takes": {1: "registers", 2: "dma", 3: "gemm"}[builtin_loader(auto.args)],
@@ -409,9 +415,7 @@ def headline(torch, dev, oracle, mm, args, operands, out):
         launch()
 
     # the clocks settle over the first few dozen launches after idle: run those before the W warm-up steps
-    for _ in range(PRE_ROLL):
-        step()
-    torch.cuda.synchronize()
+    pre_roll(step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -497,9 +501,7 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
     zeros = args.operands == "zeros"
 
     def measure(name, fn, flops, bytes_, dt, bound, nrot=1):
-        for i in range(PRE_ROLL):
-            fn(i % nrot)
-        torch.cuda.synchronize()
+        pre_roll(lambda i: fn(i % nrot))
         durs = event_times(lambda i: fn(i % nrot), reps)
         ms = region_time(lambda i: fn(i % nrot), 2 * reps)
         r = {"kernel_ms": round(ms, 4), "kernel_ms_single_mean": round(sum(durs) / len(durs), 4), "tflops": round(flops / ms / 1e9, 2), "gbs": round(bytes_ / ms / 1e6, 1)}
