@@ -482,6 +482,30 @@ def headline(torch, dev, oracle, mm, args, operands, out):
     return ok
 
 
+def graph_replay_ms(torch, bind, per_graph=100, replays=20):
+    """Per-launch ms of `per_graph` launches captured once into a HIP graph and replayed: what a launch-latency-bound
+    problem costs a caller that captures its loop (the library allocates and clears nothing, so a capture is just the
+    kernel nodes).  `bind()` returns the launch, bound to the stream that is current when it is called.  None if the
+    capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            launch = bind()
+            launch()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(per_graph):
+                launch()
+        pre_roll(lambda i: graph.replay())
+        return round(region_time(lambda i: graph.replay(), replays) / per_graph, 5)
+    except Exception as e:      # a figure beside the measurement, never a reason to fail it
+        print(f"graph replay not measured: {e}", file=sys.stderr)
+        return None
+
+
 def default_loader(conv_args):
     """Which of the conv2d kernels a launch with these arguments runs (tnx_conv_loader), by asking the library."""
     import ctypes
@@ -522,6 +546,8 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
         l1 = mm.matmul_kernel.prepare(a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg)
         r = measure("C1", lambda i: l1(), 805306368, 3407872, "f16", None)
         r["tile"] = cfg
+        r["graph_replay_ms"] = graph_replay_ms(
+            torch, lambda: mm.matmul_kernel.prepare(a, b, c, 1024, 768, 512, 512, 1, 768, 1, 768, 1, **cfg))
         if not args.no_vendor:
             cv = torch.empty_like(c)
             r["vendor_ms"] = vendor_ms(lambda i: torch.matmul(a, b, out=cv))
