@@ -174,6 +174,34 @@ def test_gemm_route_for_1x1_layers(dtype, device):
                 assert torch.equal(out, regs), (i, dtype, cfg)
 
 
+def test_seeded_random_1x1_layers_on_the_gemm_route(device):
+    """Eighty 1x1 layers drawn from a fixed seed (1-40 images, 1-300 channels either side, planes 1-30 per side, bias of
+    the tensor type, fp32 or none, the library's tile or one of the built ones): against the CPU library routine in
+    fp32, the output embedded in NaN so that a store outside it shows."""
+    rng = np.random.default_rng(77)
+    gemm_tiles = sorted({(int(f[1]), int(f[2]), int(f[3])) for f in (x.split() for x in _C.kernel_names())
+                         if f[0] == "bf16" and int(f[1]) * int(f[2]) <= 128 * 128})
+    assert len(gemm_tiles) >= 8
+    for case in range(80):
+        n, c, k = int(rng.integers(1, 41)), int(rng.integers(1, 301)), int(rng.integers(1, 301))
+        h, w = int(rng.integers(1, 31)), int(rng.integers(1, 31))
+        dtype = [torch.bfloat16, torch.float16][case % 2]
+        g = torch.Generator().manual_seed(1000 + case)
+        x = torch.randn(n, c, h, w, generator=g).to(dtype)
+        wt = (torch.randn(k, c, 1, 1, generator=g) / c ** 0.5).to(dtype)
+        b = [None, torch.randn(k, generator=g).to(dtype), torch.randn(k, generator=g)][case % 3]
+        bcout, bpix, bk = (0, 0, 0) if case % 4 == 0 else gemm_tiles[int(rng.integers(0, len(gemm_tiles)))]
+        canvas = torch.full((n * k * h * w + 48,), float("nan"), dtype=dtype, device=device)
+        out = canvas[24:24 + n * k * h * w].view(n, k, h, w)
+        conv2d_forward_kernel[(1,)](out, x.to(device), wt.to(device), None if b is None else b.to(device), n, c, h, w, k, h, w,
+                                    1, 1, 1, 1, 0, 0, 1, 1, n * h * w, k, c, BLOCK_SIZE_M=bpix, BLOCK_SIZE_N=bcout,
+                                    BLOCK_SIZE_K=bk, GROUP_SIZE_M=8, LOADER="gemm")
+        what = (case, n, c, h, w, k, dtype, None if b is None else b.dtype, bcout, bpix, bk)
+        ok, err, rel = oracle.within_tolerance(out, oracle.reference_conv2d(x, wt, b))
+        assert ok, (what, err, rel)
+        assert bool(torch.isnan(canvas[:24]).all()) and bool(torch.isnan(canvas[24 + n * k * h * w:]).all()), what
+
+
 def test_gemm_route_follows_dilation_free_geometry_only(device):
     """Dilation has no effect on a single tap; stride or padding take the layer off the GEMM route."""
     g = torch.Generator().manual_seed(5)
