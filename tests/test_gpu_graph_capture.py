@@ -32,7 +32,7 @@ def test_a_captured_sequence_replays_with_the_eager_bits(device, monkeypatch):
         h = tritonix_amd.triton_matmul(a, b)
         return [h, tritonix_amd.triton_matmul(h, b.t()),            # a launch fed by a launch; k-contiguous B
                 tritonix_amd.matmul_splitk(xs, ws), tritonix_amd.swiglu(xg, w12), tritonix_amd.triton_matmul(ai, bi),
-                conv2d_forward(img, w1, bias, config=dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0)),
+                conv2d_forward(img, w1, bias),                      # TRITONIX_AUTOTUNE=0: the library's choice, untimed
                 conv2d_forward(img, w3, None, (1, 1), (1, 1), (1, 1),
                                config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64)),
                 conv2d_forward(img, w3, None, (2, 2), (1, 1), (1, 1),

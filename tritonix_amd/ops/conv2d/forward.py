@@ -11,6 +11,7 @@ gfx950 has no TF32 matrix instruction.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -221,7 +222,7 @@ def conv2d_forward(
     """conv2d forward on the HIP kernel; same arguments and result as tritonix/ops/conv2d/forward.py:202-311.
 
     ``config=None`` times the candidate tiles once per problem key and remembers the fastest, as the reference
-    does; ``config={"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K"[, "GROUP_SIZE_M"][, "LOADER"]}`` launches that tile
+    does (with ``TRITONIX_AUTOTUNE=0`` in the environment it launches the library's built-in choice instead); ``config={"BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K"[, "GROUP_SIZE_M"][, "LOADER"]}`` launches that tile
     (all three sizes 0: the library's own choice; ``LOADER`` is "auto", "registers", "dma" or "gemm").
     Returns a new [N, C_OUT, H_OUT, W_OUT] tensor of the input's dtype."""
     assert input.is_contiguous(), "Input must be contiguous NCHW"
@@ -243,6 +244,8 @@ def conv2d_forward(
             stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], gemm_m, gemm_n, gemm_k,
             BLOCK_SIZE_M=bm, BLOCK_SIZE_N=bn, BLOCK_SIZE_K=bk, GROUP_SIZE_M=g, USE_TF32=use_tf32, LOADER=loader)
 
+    if config is None and os.environ.get("TRITONIX_AUTOTUNE", "1") in ("0", "false", "False"):
+        config = dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0)      # no timing runs: the library's own choice
     if config is None:
         key = (n, c_in, h_in, w_in, c_out, r, s, stride, padding, dilation, input.dtype)
         cfg = _CONV_FWD_CONFIG_CACHE.get(key)
