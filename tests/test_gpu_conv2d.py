@@ -191,15 +191,21 @@ def test_seeded_random_1x1_layers_on_the_gemm_route(device):
         wt = (torch.randn(k, c, 1, 1, generator=g) / c ** 0.5).to(dtype)
         b = [None, torch.randn(k, generator=g).to(dtype), torch.randn(k, generator=g)][case % 3]
         bcout, bpix, bk = (0, 0, 0) if case % 4 == 0 else gemm_tiles[int(rng.integers(0, len(gemm_tiles)))]
-        canvas = torch.full((n * k * h * w + 48,), float("nan"), dtype=dtype, device=device)
-        out = canvas[24:24 + n * k * h * w].view(n, k, h, w)
-        conv2d_forward_kernel[(1,)](out, x.to(device), wt.to(device), None if b is None else b.to(device), n, c, h, w, k, h, w,
-                                    1, 1, 1, 1, 0, 0, 1, 1, n * h * w, k, c, BLOCK_SIZE_M=bpix, BLOCK_SIZE_N=bcout,
-                                    BLOCK_SIZE_K=bk, GROUP_SIZE_M=8, LOADER="gemm")
-        what = (case, n, c, h, w, k, dtype, None if b is None else b.dtype, bcout, bpix, bk)
+        # every third case: output, input and weight start an odd number of elements into their allocations
+        off = 25 if case % 3 == 1 else 24
+        canvas = torch.full((n * k * h * w + 2 * off,), float("nan"), dtype=dtype, device=device)
+        out = canvas[off:off + n * k * h * w].view(n, k, h, w)
+        xd = torch.full((x.numel() + off,), float("nan"), dtype=dtype, device=device)
+        xd[off:].copy_(x.reshape(-1))
+        wd = torch.full((wt.numel() + off,), float("nan"), dtype=dtype, device=device)
+        wd[off:].copy_(wt.reshape(-1))
+        conv2d_forward_kernel[(1,)](out, xd[off:].view(n, c, h, w), wd[off:].view(k, c, 1, 1), None if b is None else b.to(device),
+                                    n, c, h, w, k, h, w, 1, 1, 1, 1, 0, 0, 1, 1, n * h * w, k, c, BLOCK_SIZE_M=bpix,
+                                    BLOCK_SIZE_N=bcout, BLOCK_SIZE_K=bk, GROUP_SIZE_M=8, LOADER="gemm")
+        what = (case, n, c, h, w, k, dtype, None if b is None else b.dtype, bcout, bpix, bk, off)
         ok, err, rel = oracle.within_tolerance(out, oracle.reference_conv2d(x, wt, b))
         assert ok, (what, err, rel)
-        assert bool(torch.isnan(canvas[:24]).all()) and bool(torch.isnan(canvas[24 + n * k * h * w:]).all()), what
+        assert bool(torch.isnan(canvas[:off]).all()) and bool(torch.isnan(canvas[off + n * k * h * w:]).all()), what
 
 
 def test_gemm_route_follows_dilation_free_geometry_only(device):
