@@ -211,7 +211,8 @@ def sustain(step, seconds, flops):
 SWEEP_SHAPES = [(1, 4096, 4096), (8, 14336, 4096), (32, 4096, 14336), (64, 8192, 8192), (128, 8192, 8192),
                 (512, 4096, 4096), (1024, 1024, 1024), (2048, 2048, 512), (2048, 2048, 2048), (1024, 4096, 4096),
                 (3072, 3072, 3072), (4096, 4096, 4096),
-                (4096, 4096, 4104), (4096, 4100, 4096), (4100, 4096, 4096)]
+                (4096, 4096, 4104), (4096, 4100, 4096), (4100, 4096, 4096),
+                (512, 4096, 4096, "kc"), (4096, 4096, 4096, "kc"), (4096, 14336, 4096, "kc"), (8192, 8192, 8192, "kc")]
 
 
 def shape_sweep(torch, dev, mm):
@@ -219,20 +220,24 @@ def shape_sweep(torch, dev, mm):
     (`prepare`), B rotated over several copies so that skinny shapes stream it from HBM; the vendor's GEMM on the
     same operands beside it."""
     rows = []
-    for m, n, k in SWEEP_SHAPES:
+    for m, n, k, *layout in SWEEP_SHAPES:
         g = torch.Generator("cpu").manual_seed(m + n + k)
         a = (torch.randn(m, k, generator=g) / k ** 0.5).bfloat16().to(dev)
-        b0 = torch.randn(k, n, generator=g).bfloat16()
-        bs = [b0.to(dev).clone() for _ in range(4 if k * n * 2 < 300e6 else 2)]
+        if layout:      # "kc": B is the transposed view of an [n, k] weight, the `x @ w.t()` of a linear layer
+            b0 = torch.randn(n, k, generator=g).bfloat16()
+            bs = [b0.to(dev).clone().t() for _ in range(4 if k * n * 2 < 300e6 else 2)]
+        else:
+            b0 = torch.randn(k, n, generator=g).bfloat16()
+            bs = [b0.to(dev).clone() for _ in range(4 if k * n * 2 < 300e6 else 2)]
         cfg = mm.default_config(a, bs[0])
         kern = mm.gemm_splitk_kernel if cfg.get("split_k", 1) > 1 else mm.matmul_kernel
         c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
-        ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), 1, n, 1, **cfg) for b in bs]
+        ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), b.stride(1), n, 1, **cfg) for b in bs]
         pre_roll(lambda i: ls[i % len(ls)]())
         ours = region_time(lambda i: ls[i % len(ls)](), 50)
         pre_roll(lambda i: torch.matmul(a, bs[i % len(bs)], out=c))
         vendor = region_time(lambda i: torch.matmul(a, bs[i % len(bs)], out=c), 50)
-        rows.append({"shape": [m, n, k], "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),
+        rows.append({"shape": [m, n, k], "b_layout": "k-contiguous" if layout else "row-major", "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),
                      "gbs": round(2.0 * (m * k + k * n + m * n) / ours / 1e6, 1), "vendor_ms": round(vendor, 4),
                      "config": cfg})
     return rows
