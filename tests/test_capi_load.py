@@ -175,8 +175,14 @@ def test_default_config_of_the_benchmark_shapes():
     assert pick(_C.BF16, _C.BF16, 16, 4096, 14336) == (64, 128, 64, 8, 3, 8, 0)
     # 576 tiles of 256x256 are 2.25 waves of 256 CUs: the last 64 tiles are cut four ways
     assert pick(_C.BF16, _C.BF16, 6144, 6144, 6144) == (256, 256, 64, 4, 2, 4, 64)
-    # 400 tiles: 144 trailing tiles cannot be cut without spilling into another wave
-    assert pick(_C.BF16, _C.BF16, 5120, 5120, 8192) == (256, 256, 64, 4, 2, 1, 0)
+    # 400 tiles of 256x256 are 1.56 waves and the 144 trailing ones cannot be cut without spilling into another wave;
+    # 729 tiles of 192x192 are 2.85 (measured 326-331 us against 348-353)
+    assert pick(_C.BF16, _C.BF16, 5120, 5120, 8192) == (192, 192, 64, 8, 3, 1, 0)
+    assert pick(_C.I8, _C.I32, 5120, 5120, 8192) == (256, 256, 128, 4, 2, 1, 0)            # no 192-wide int8 tile
+    picked.pop()
+    # 144 tiles of 256x256 leave 112 CUs idle; 256 tiles of 192x192 are one full wave
+    assert pick(_C.BF16, _C.BF16, 3072, 3072, 3072) == (192, 192, 64, 8, 3, 1, 0)
+    picked.pop()
     # grids of at least 16 x 16 uncut tiles are walked in super-block order; nothing is made persistent by default
     assert picked == [_C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, 0, 0, 0, _C.SCHED_SUPERBLOCK]
 

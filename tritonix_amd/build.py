@@ -51,7 +51,7 @@ def tile_valid(es, bm, bn, bk, nw, stages):
     if (bk * es) % kb or bk * es < kb:
         return False
     cpr_a, cpr_b = bk * es // 16, bn * es // 16
-    if cpr_a < 4 or cpr_b < 8:
+    if cpr_a < 4 or cpr_b < 8 or cpr_b % 8:
         return False
     a_bytes, b_bytes = bm * bk * es, bk * bn * es
     if a_bytes % 1024 or b_bytes % 1024:
@@ -101,6 +101,13 @@ def instance_list(quick=False):
                             # element-wise (any stride / ragged K) variants only for two small tiles
                             generic = nw == 4 and st == 2 and bk == bks[1] and (bm, bn) in ((128, 128), (64, 128))
                             out.append((dt, bm, bn, bk, nw, st, generic))
+        # 192 x 192: sixteen tiles per 3072 where the 256-wide tile has twelve -- problems whose sides are multiples of
+        # 192 but leave a round of 256x256 tiles half empty (3072^3 is 144 of those on 256 CUs, and 256 of these)
+        if es == 2 and not quick:
+            for nw in (4, 8):
+                for st in (2, 3):
+                    assert tile_valid(es, 192, 192, 64, nw, st)
+                    out.append((dt, 192, 192, 64, nw, st, False))
     return out
 
 

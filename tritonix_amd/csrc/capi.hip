@@ -403,9 +403,11 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   // reads back at about 60 GB/s.  Three shapes of launch are priced per tile: uncut; every tile cut (only when
   // the tiles alone leave CUs idle); only the tiles of the partial wave cut (tail_tiles).  Slices never get
   // shorter than eight K slabs.
-  static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}};
-  static const double rate[] = {1.0, 0.9, 0.75, 0.5, 0.35};
-  const int ncand = es == 1 ? 4 : 5;   // int8 rows of a 64-wide B tile are too short for the transposing read
+  // (the sixth, 192x192, exists for the 16-bit types: it is what divides sides like 1536, 3072 or 4608 into whole
+  // rounds -- 3072^3 is 144 tiles of 256x256 on 256 CUs, and 256 of these: measured 62 -> 47 us)
+  static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}, {192, 192, 3, 8}};
+  static const double rate[] = {1.0, 0.9, 0.75, 0.5, 0.35, 0.92};
+  const int ncand = es == 1 ? 4 : 6;   // int8 rows of a 64-wide B tile are too short for the transposing read
   const double cu_flops = 5.5e12 * (es == 1 ? 1.7 : 1.0);          // per CU with the largest tile
   const double launch = 3e-6, handover = 9e-6, readback = 60e9;
   const int64_t kt = (a->k + bk - 1) / bk;

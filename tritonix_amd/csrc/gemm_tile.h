@@ -366,7 +366,7 @@ struct TileCfg {
   static constexpr int ACC_N = (MI == 32) ? 16 : 4;
   static constexpr bool VALID =
       (WTM % 16 == 0) && (WTN % 16 == 0) && (BK * ES) % KB == 0 && KSTEPS >= 1 && CPR_A >= 4 &&
-      (ES == 2 ? CPR_B >= 8 : CPR_B >= 8) && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
+      CPR_B >= 8 && CPR_B % 8 == 0 && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
       A_LOADS % NW == 0 && B_LOADS % NW == 0 && LDS_BYTES <= 163840 && TM * TN * ACC_N <= 256 && (STAGES - 2) * LPW <= 63 && STAGES >= 2;
 
   // chunk-index XOR applied to row `row` of the A slab.  A fragment read is one ds_read_b128 with lane = 16 * kg +
@@ -387,11 +387,11 @@ struct TileCfg {
   static __host__ __device__ constexpr int swzB(int row) {
     if (ES == 2) {
       const int pass = MI == 16 ? (((row >> 3) ^ (row >> 4)) & 1) << 1 : 0;
-      if (CPR_B >= 16) { int k = row & 3; return ((2 * k + (k >> 1)) << 1) ^ pass; }
-      return ((row & 3) << 1) ^ pass;
+      if (CPR_B % 16 == 0) { int k = row & 3; return ((2 * k + (k >> 1)) << 1) ^ pass; }
+      return ((row & 3) << 1) ^ pass;       // stays inside a group of 8 chunks: also for rows of 24 chunks (BN = 192)
     } else {
       const int pass = MI == 16 ? ((row >> 4) ^ (row >> 5)) & 1 : 0;
-      if (CPR_B >= 16) { int k = row & 7; return (2 * k + (k >> 2)) ^ pass; }
+      if (CPR_B % 16 == 0) { int k = row & 7; return (2 * k + (k >> 2)) ^ pass; }
       return (row & 7) ^ pass;
     }
   }
@@ -460,10 +460,16 @@ struct SliceSrc {
 // Sum of the split-K slices of one row-block of a wave, group by group, into the wave's LDS
 // strip (same places the accumulators of an uncut tile go).  ZB slices of G = 32 / ZB groups
 // are fetched together; slices are added in slice order whatever ZB is.
+// largest batch of groups <= cap that divides the nq groups of a row-block (nq is 6 for the 192-wide tiles)
+constexpr int slice_batch(int nq, int cap) {
+  int g = cap < nq ? cap : nq;
+  while (nq % g) --g;
+  return g;
+}
 template <class ACC4, int ZB, int NQ, int MI, int NGRP>
 __device__ __forceinline__ void sum_slices(__amdgpu_buffer_rsrc_t win, uint32_t q0, const SliceSrc& src, uint32_t wbase,
                                            bool row_ok) {
-  constexpr int G = (32 / ZB) < NQ ? (32 / ZB) : NQ;
+  constexpr int G = slice_batch(NQ, 32 / ZB);
   static_assert(NQ % G == 0, "groups per row-block must be a multiple of the batch");
 #pragma unroll 1
   for (int jg0 = 0; jg0 < NQ; jg0 += G) {

@@ -88,7 +88,7 @@ template <class T, class C> struct BtLaunch<T, C, true> {
 template <class C> constexpr bool conv_ok() {
   return C::ES == 2 && C::NW == 8 && C::KSTEPS * C::TM * C::TN >= 16 &&
          C::KSTEPS * C::TM * C::TN / 2 > C::B_LPW + (C::KSTEPS * C::TM * C::TN >= 32 ? 6 : 3) + 1 && C::STAGES == 3 && C::BK == 64 &&
-         C::BM >= 128 && C::BN >= 128 && C::TM * C::TN * C::ACC_N <= 128;
+         C::BM >= 128 && C::BN >= 128 && C::TM * C::TN * C::ACC_N <= 128 && (C::NW * 64) % C::CPR_B == 0;
 }
 template <class T, class C, bool OK = conv_ok<C>()> struct ConvLaunch {
   static constexpr launch_fn fn = nullptr;
