@@ -198,3 +198,43 @@ def test_atomic_reduction_of_split_k_slices(device):
         c = torch.full((100, 264), 7, device=device, dtype=torch.bfloat16)
         launch(matmul_kernel, ar.to(device), br.to(device), c, cfg(128, 128, 64, 4, 2, split_k=3, atomic_reduce=1))
         assert oracle.within_tolerance(c, oracle.reference_matmul(ar, br))[0]
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the 192x192 tile: rows of 24 chunks in the B slab, 6 x 6 MFMA tiles per wave (four waves) -- the one tile whose
+# sides are not powers of two
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda v: str(v).replace("torch.", ""))
+@pytest.mark.parametrize("waves,stages", [(4, 2), (4, 3), (8, 2), (8, 3)])
+def test_the_192_tile_gives_the_bits_of_the_128_tile(device, dtype, waves, stages):
+    """Every tile with a 64-deep K slab adds the same products in the same order, so the results must agree bit for bit:
+    whole and ragged problems, the super-block order, K cut for all tiles and for the last ones only, k-contiguous B,
+    the gated epilogue."""
+    from tritonix_amd.ops.matmul import gemm_splitk_kernel
+
+    for (m, n, k) in [(384, 576, 256), (1000, 1100, 520), (3072, 3072, 512), (190, 194, 64), (2880, 200, 1024)]:
+        g = torch.Generator("cpu").manual_seed(m + n + k)
+        a = torch.randn(m, k, generator=g).to(dtype)
+        b = (torch.randn(k, n, generator=g) / k ** 0.5).to(dtype)
+        ad, bd = a.to(device), b.to(device)
+        want = gemm(ad, bd, cfg(128, 128, 64, 4, 2))
+        rows = torch.arange(0, m, max(1, m // 16))
+        assert oracle.within_tolerance(want[rows.to(device)], oracle.reference_matmul(a[rows], b))[0]
+        tile = (192, 192, 64, waves, stages)
+        assert torch.equal(gemm(ad, bd, cfg(*tile)), want), (m, n, k, "plain")
+        assert torch.equal(gemm(ad, bd, cfg(*tile, superblock=1)), want), (m, n, k, "super-block order")
+        wt = bd.t().contiguous()                                   # B as the transposed view of an [n, k] weight
+        assert torch.equal(gemm(ad, wt.t(), cfg(*tile)), want), (m, n, k, "k-contiguous B")
+        if k >= 512:
+            # K cut: fp32 partial sums are added in slice order, not in one chain; compare with the same cut on the 128 tile
+            tiles = cdiv(m, 192) * cdiv(n, 192)
+            for extra in (dict(split_k=2), dict(split_k=4, tail_tiles=min(3, tiles))):
+                c = torch.full((m, n), 7, device=device, dtype=dtype)
+                launch(gemm_splitk_kernel, ad, bd, c, cfg(*tile, **extra))
+                assert oracle.within_tolerance(c[rows.to(device)], oracle.reference_matmul(a[rows], b))[0], (m, n, k, extra)
+        if n % 2 == 0:
+            z = torch.full((m, n // 2), 7, device=device, dtype=dtype)
+            z128 = torch.full((m, n // 2), 7, device=device, dtype=dtype)
+            launch(glu_kernel, ad, bd, z, cfg(*tile), activation="silu")
+            launch(glu_kernel, ad, bd, z128, cfg(128, 128, 64, 4, 2), activation="silu")
+            assert torch.equal(z, z128), (m, n, k, "gated")
