@@ -440,7 +440,8 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   // 16-bit problems with a short K loop (at most 64 slabs per tile) spend a visible share of every tile outside
   // it; two waves per SIMD cover that better than one (measured on 4096 x 28672 x 4096, gated: +2.4 %), at the
   // price of half again as many LDS reads, which is what loses on the long, power-limited 8192^3 loops.
-  if (es == 2 && bi == 0 && bs == 1 && kt <= 64) a->num_warps = 8;
+  // (cut tiles too: 4096 x 5120 x 4096 with its last 64 tiles cut, 155 -> 140 us)
+  if (es == 2 && bi == 0 && kt <= 64) a->num_warps = 8;
   a->split_k = bs;
   a->tail_tiles = btail;
   // Grids of several rounds of 256 tiles in both directions: the super-block order keeps what one round reads
