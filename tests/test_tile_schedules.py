@@ -201,12 +201,13 @@ def test_atomic_reduction_of_split_k_slices(device):
 
 
 # ---------------------------------------------------------------------------------------------------------------------
-# the 192x192 tile: rows of 24 chunks in the B slab, 6 x 6 MFMA tiles per wave (four waves) -- the one tile whose
+# the 192x192, 192x256 and 256x192 tiles: rows of 24 chunks in the B slab, 6 MFMA tiles across a wave -- the tiles whose
 # sides are not powers of two
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda v: str(v).replace("torch.", ""))
-@pytest.mark.parametrize("waves,stages", [(4, 2), (4, 3), (8, 2), (8, 3)])
-def test_the_192_tile_gives_the_bits_of_the_128_tile(device, dtype, waves, stages):
+@pytest.mark.parametrize("bm,bn,waves,stages", [(192, 192, 4, 2), (192, 192, 4, 3), (192, 192, 8, 2), (192, 192, 8, 3),
+                                                (192, 256, 4, 2), (192, 256, 8, 2), (256, 192, 4, 2), (256, 192, 8, 2)])
+def test_the_192_tiles_give_the_bits_of_the_128_tile(device, dtype, bm, bn, waves, stages):
     """Every tile with a 64-deep K slab adds the same products in the same order, so the results must agree bit for bit:
     whole and ragged problems, the super-block order, K cut for all tiles and for the last ones only, k-contiguous B,
     the gated epilogue."""
@@ -220,14 +221,14 @@ def test_the_192_tile_gives_the_bits_of_the_128_tile(device, dtype, waves, stage
         want = gemm(ad, bd, cfg(128, 128, 64, 4, 2))
         rows = torch.arange(0, m, max(1, m // 16))
         assert oracle.within_tolerance(want[rows.to(device)], oracle.reference_matmul(a[rows], b))[0]
-        tile = (192, 192, 64, waves, stages)
+        tile = (bm, bn, 64, waves, stages)
         assert torch.equal(gemm(ad, bd, cfg(*tile)), want), (m, n, k, "plain")
         assert torch.equal(gemm(ad, bd, cfg(*tile, superblock=1)), want), (m, n, k, "super-block order")
         wt = bd.t().contiguous()                                   # B as the transposed view of an [n, k] weight
         assert torch.equal(gemm(ad, wt.t(), cfg(*tile)), want), (m, n, k, "k-contiguous B")
         if k >= 512:
             # K cut: fp32 partial sums are added in slice order, not in one chain; compare with the same cut on the 128 tile
-            tiles = cdiv(m, 192) * cdiv(n, 192)
+            tiles = cdiv(m, bm) * cdiv(n, bn)
             for extra in (dict(split_k=2), dict(split_k=4, tail_tiles=min(3, tiles))):
                 c = torch.full((m, n), 7, device=device, dtype=dtype)
                 launch(gemm_splitk_kernel, ad, bd, c, cfg(*tile, **extra))

@@ -103,11 +103,15 @@ def instance_list(quick=False):
                             out.append((dt, bm, bn, bk, nw, st, generic))
         # 192 x 192: sixteen tiles per 3072 where the 256-wide tile has twelve -- problems whose sides are multiples of
         # 192 but leave a round of 256x256 tiles half empty (3072^3 is 144 of those on 256 CUs, and 256 of these)
+        # 192 x 256 and 256 x 192 (two ring slots fit): 4096 x 2560 is 160 tiles of 256x256 and 220 / 224 of these
         if es == 2 and not quick:
             for nw in (4, 8):
                 for st in (2, 3):
                     assert tile_valid(es, 192, 192, 64, nw, st)
                     out.append((dt, 192, 192, 64, nw, st, False))
+                for bm, bn in ((192, 256), (256, 192)):
+                    assert tile_valid(es, bm, bn, 64, nw, 2)
+                    out.append((dt, bm, bn, 64, nw, 2, False))
     return out
 
 

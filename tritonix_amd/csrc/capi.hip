@@ -405,9 +405,13 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   // shorter than eight K slabs.
   // (the sixth, 192x192, exists for the 16-bit types: it is what divides sides like 1536, 3072 or 4608 into whole
   // rounds -- 3072^3 is 144 tiles of 256x256 on 256 CUs, and 256 of these: measured 62 -> 47 us)
-  static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}, {192, 192, 3, 8}};
-  static const double rate[] = {1.0, 0.9, 0.75, 0.5, 0.35, 0.92};
-  const int ncand = es == 1 ? 4 : 6;   // int8 rows of a 64-wide B tile are too short for the transposing read
+  // (192x256 and 256x192 likewise: 4096 x 2560 x 8192 is 160 tiles of 256x256, 0.63 of a round, and 220 of 192x256:
+  // measured 141 -> 128 us; their rate lies between what they reach against 256x256 on 8192^3, 0.86, and on
+  // launches of a round or two at K = 4096, where they run at the full 0.75 of its tile time)
+  static const int cand[][4] = {{256, 256, 2, 4}, {256, 128, 3, 4}, {128, 128, 3, 4}, {64, 128, 3, 4}, {64, 64, 4, 4}, {192, 192, 3, 8},
+                                {192, 256, 2, 8}, {256, 192, 2, 8}};
+  static const double rate[] = {1.0, 0.9, 0.75, 0.5, 0.35, 0.92, 0.9, 0.9};
+  const int ncand = es == 1 ? 4 : 8;   // int8 rows of a 64-wide B tile are too short for the transposing read
   const double cu_flops = 5.5e12 * (es == 1 ? 1.7 : 1.0);          // per CU with the largest tile
   const double launch = 3e-6, handover = 9e-6, readback = 60e9;
   const int64_t kt = (a->k + bk - 1) / bk;
