@@ -420,12 +420,18 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   auto offer = [&](double t, int i, int s, int tail) {
     if (t < best * 0.97) { best = t; bi = i; bs = s; btail = tail; }   // ties go to the earlier (larger, less cut) choice
   };
+  // (The 0.75 holds for nearly full last waves of the large tiles too: 220 tiles of 192x256 on 256 CUs took 0.80 of a
+  // full wave's time; a cost that rises with the fill, 0.7 + 0.3 * rem / 256, was tried on 382 shapes and moved a
+  // third of 75 choices for the worse by up to 20 %.  The tiles up to 128x128 do not load the power limit, so their
+  // partial wave runs no faster than a full one: 128 tiles of 64x128 took 0.91 of the modelled full wave where 256
+  // tiles of 64x64 took 1.0 of theirs; they are priced at 0.9.)
   for (int i = 0; i < ncand; ++i) {
     const int64_t tiles = ((a->m + cand[i][0] - 1) / cand[i][0]) * ((a->n + cand[i][1] - 1) / cand[i][1]);
     const double tile_t = 2.0 * cand[i][0] * cand[i][1] * (double)a->k / (cu_flops * rate[i]);
     const double slice_bytes = (double)cand[i][0] * cand[i][1] * 4;
+    const double part = (i >= 2 && i <= 4) ? 0.9 : 0.75;            // cost of a last, partial wave (see above)
     const int64_t full = tiles / cus, rem = tiles % cus;
-    offer((double)full * tile_t + (rem ? 0.75 * tile_t : 0.0) + launch, i, 1, 0);
+    offer((double)full * tile_t + (rem ? part * tile_t : 0.0) + launch, i, 1, 0);
     for (int s = 2; s <= 16; s *= 2) {
       if (kt / s < 8) break;
       if (full == 0 && tiles * s <= cus)                             // every tile cut (one wave at most)
