@@ -274,3 +274,44 @@ def test_measurement_probes_launch_and_finish(device):
         assert lib.tnx_probe_lds(op, table, 4, scratch.data_ptr(), 512, stream) == _C.OK, name
         torch.cuda.synchronize()
         assert scratch[:64].view(torch.int32).tolist() == offs      # the table the kernel read
+
+
+def test_built_in_choice_on_seeded_random_problems(device, monkeypatch):
+    """150 problems from a fixed seed (round sizes, ragged sizes, thin and wide, all three types, every fifth with a
+    k-contiguous B) through ``triton_matmul`` with the library's own tile choice: whatever tile, K cut or tail cut it
+    names must give the right product (int8 exactly)."""
+    import random
+
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    mm._matmul_cfg.clear()
+    rnd = random.Random(5)
+    picked = set()
+    for case in range(150):
+        kind = case % 4
+        if kind == 0:
+            m, n, k = (rnd.choice([128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 2560, 3072]) for _ in range(3))
+        elif kind == 1:
+            m, n, k = rnd.randint(1, 700), rnd.randint(1, 3000), rnd.randint(1, 3000)
+        elif kind == 2:
+            m, n, k = rnd.randint(100, 3000), rnd.randint(100, 3000), 64 * rnd.randint(1, 64)
+        else:
+            m, n, k = 8 * rnd.randint(1, 400), 8 * rnd.randint(1, 400), 8 * rnd.randint(1, 600)
+        dt = [torch.bfloat16, torch.float16, torch.int8][case % 3]
+        g = torch.Generator(device=device).manual_seed(case)
+        if dt == torch.int8:
+            a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device=device, generator=g)
+            b = torch.randint(-127, 128, (k, n), dtype=torch.int8, device=device, generator=g)
+        else:
+            a = torch.randn(m, k, device=device, generator=g).to(dt)
+            b = (torch.randn(k, n, device=device, generator=g) / k ** 0.5).to(dt)
+        if case % 5 == 4:
+            b = b.t().contiguous().t()
+        cfg = mm.default_config(a, b)
+        picked.add((cfg["block_m"], cfg["block_n"], cfg.get("split_k", 1) > 1))
+        out = tritonix_amd.triton_matmul(a, b)
+        what = (case, m, n, k, dt, cfg)
+        if dt == torch.int8:
+            assert torch.equal(out.double(), a.double() @ b.double()), what
+        else:
+            assert oracle.within_tolerance(out, a.float() @ b.float())[0], what
+    assert len(picked) >= 6, picked
