@@ -112,6 +112,11 @@ def instance_list(quick=False):
                 for bm, bn in ((192, 256), (256, 192)):
                     assert tile_valid(es, bm, bn, 64, nw, 2)
                     out.append((dt, bm, bn, 64, nw, 2, False))
+        # int8: 192 x 256 only (rows of 192 bytes in the B slab have no swizzle)
+        if es == 1 and not quick:
+            for nw in (4, 8):
+                assert tile_valid(es, 192, 256, 128, nw, 2)
+                out.append((dt, 192, 256, 128, nw, 2, False))
     return out
 
 
