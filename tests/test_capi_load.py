@@ -178,7 +178,7 @@ def test_default_config_of_the_benchmark_shapes():
     # 400 tiles of 256x256 are 1.56 waves and the 144 trailing ones cannot be cut without spilling into another wave;
     # 729 tiles of 192x192 are 2.85 (measured 326-331 us against 348-353)
     assert pick(_C.BF16, _C.BF16, 5120, 5120, 8192) == (192, 192, 64, 8, 3, 1, 0)
-    assert pick(_C.I8, _C.I32, 5120, 5120, 8192) == (256, 256, 128, 4, 2, 1, 0)            # no 192-wide int8 tile
+    assert pick(_C.I8, _C.I32, 5120, 5120, 8192) == (192, 192, 128, 8, 3, 1, 0)            # int8 has the 192 tiles too
     picked.pop()
     # 144 tiles of 256x256 leave 112 CUs idle; 256 tiles of 192x192 are one full wave
     assert pick(_C.BF16, _C.BF16, 3072, 3072, 3072) == (192, 192, 64, 8, 3, 1, 0)

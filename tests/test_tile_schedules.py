@@ -242,8 +242,9 @@ def test_the_192_tiles_give_the_bits_of_the_128_tile(device, dtype, bm, bn, wave
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("bm,bn,stages", [(192, 256, 2), (256, 192, 2), (192, 192, 2), (192, 192, 3)])
 @pytest.mark.parametrize("waves", [4, 8])
-def test_the_int8_192x256_tile_is_exact(device, waves):
+def test_the_int8_192_tiles_are_exact(device, waves, bm, bn, stages):
     for (m, n, k) in [(384, 512, 256), (1000, 1100, 520), (3072, 1024, 1024), (190, 200, 128)]:
         g = torch.Generator("cpu").manual_seed(m + n + k)
         a = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8)
@@ -252,5 +253,5 @@ def test_the_int8_192x256_tile_is_exact(device, waves):
         want = gemm(ad, bd, cfg(128, 128, 128, 4, 2))
         rows = torch.arange(0, m, max(1, m // 16))
         assert torch.equal(want[rows.to(device)].cpu(), oracle.reference_matmul(a[rows], b))
-        assert torch.equal(gemm(ad, bd, cfg(192, 256, 128, waves, 2)), want), (m, n, k)
-        assert torch.equal(gemm(ad, bd, cfg(192, 256, 128, waves, 2, superblock=1)), want), (m, n, k, "super-block order")
+        assert torch.equal(gemm(ad, bd, cfg(bm, bn, 128, waves, stages)), want), (m, n, k)
+        assert torch.equal(gemm(ad, bd, cfg(bm, bn, 128, waves, stages, superblock=1)), want), (m, n, k, "super-block order")

@@ -51,7 +51,7 @@ def tile_valid(es, bm, bn, bk, nw, stages):
     if (bk * es) % kb or bk * es < kb:
         return False
     cpr_a, cpr_b = bk * es // 16, bn * es // 16
-    if cpr_a < 4 or cpr_b < 8 or cpr_b % 8:
+    if cpr_a < 4 or cpr_b < 8 or cpr_b % (4 if es == 1 else 8):
         return False
     a_bytes, b_bytes = bm * bk * es, bk * bn * es
     if a_bytes % 1024 or b_bytes % 1024:
@@ -112,11 +112,14 @@ def instance_list(quick=False):
                 for bm, bn in ((192, 256), (256, 192)):
                     assert tile_valid(es, bm, bn, 64, nw, 2)
                     out.append((dt, bm, bn, 64, nw, 2, False))
-        # int8: 192 x 256 only (rows of 192 bytes in the B slab have no swizzle)
         if es == 1 and not quick:
             for nw in (4, 8):
-                assert tile_valid(es, 192, 256, 128, nw, 2)
-                out.append((dt, 192, 256, 128, nw, 2, False))
+                for st in (2, 3):
+                    assert tile_valid(es, 192, 192, 128, nw, st)
+                    out.append((dt, 192, 192, 128, nw, st, False))
+                for bm, bn in ((192, 256), (256, 192)):
+                    assert tile_valid(es, bm, bn, 128, nw, 2)
+                    out.append((dt, bm, bn, 128, nw, 2, False))
     return out
 
 

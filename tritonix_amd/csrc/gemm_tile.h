@@ -366,7 +366,7 @@ struct TileCfg {
   static constexpr int ACC_N = (MI == 32) ? 16 : 4;
   static constexpr bool VALID =
       (WTM % 16 == 0) && (WTN % 16 == 0) && (BK * ES) % KB == 0 && KSTEPS >= 1 && CPR_A >= 4 &&
-      CPR_B >= 8 && CPR_B % 8 == 0 && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
+      CPR_B >= 8 && CPR_B % (ES == 1 ? 4 : 8) == 0 && A_BYTES % 1024 == 0 && B_BYTES % 1024 == 0 &&
       A_LOADS % NW == 0 && B_LOADS % NW == 0 && LDS_BYTES <= 163840 && TM * TN * ACC_N <= 256 && (STAGES - 2) * LPW <= 63 && STAGES >= 2;
 
   // chunk-index XOR applied to row `row` of the A slab.  A fragment read is one ds_read_b128 with lane = 16 * kg +
@@ -392,7 +392,8 @@ struct TileCfg {
     } else {
       const int pass = MI == 16 ? ((row >> 4) ^ (row >> 5)) & 1 : 0;
       if (CPR_B % 16 == 0) { int k = row & 7; return (2 * k + (k >> 2)) ^ pass; }
-      return (row & 7) ^ pass;
+      if (CPR_B % 8 == 0) return (row & 7) ^ pass;
+      return (row & 3) ^ pass;              // rows of 12 chunks (BN = 192): stays inside a group of 4
     }
   }
 };
