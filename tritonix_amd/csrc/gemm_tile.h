@@ -393,7 +393,10 @@ struct TileCfg {
       const int pass = MI == 16 ? ((row >> 4) ^ (row >> 5)) & 1 : 0;
       if (CPR_B % 16 == 0) { int k = row & 7; return (2 * k + (k >> 2)) ^ pass; }
       if (CPR_B % 8 == 0) return (row & 7) ^ pass;
-      return (row & 3) ^ pass;              // rows of 12 chunks (BN = 192): stays inside a group of 4
+      // Rows of 12 chunks (BN = 192), 192 bytes: consecutive rows already start 48 banks apart, so the 8 rows of a
+      // 16-lane group only collide with the row 4 below, and the two groups of a pass (rows r and r + 16) with each
+      // other: one XOR bit for each, inside a group of 4 chunks.
+      return ((row >> 2) & 1) | (((row >> 4) & 1) << 1);
     }
   }
 };
