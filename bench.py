@@ -21,12 +21,6 @@ Switches for profiling and for the clock / power evidence:
   --operands zeros   all-zero operands of the same shapes: the same instruction stream without data-dependent
                      switching power, so the shader clock stays at its maximum (results are then trivially zero)
   --splitk-reduce atomic   C3 with the K slices added by fp32 atomics instead of the ordered hand-over (for the A/B)
-  --mfma-ceiling     time tnx_probe_mfma: nothing but MFMAs on register operands, 16x16 and 32x32 tiles, random and
-                     all-zero operands; what the pipes sustain on this board before any data is moved ("mfma_ceiling")
-  --shape-sweep      the built-in tile choice on a ladder of other bf16 shapes (GEMV to 4096^3, aligned and ragged)
-                     beside the vendor library's GEMM on the same operands ("shape_sweep")
-  --conv1x1-sweep    the 1x1 layers of a ResNet-50 (bf16, batch 8 / 32 / 128) on the GEMM route and on the conv2d
-                     kernel the library would otherwise take, built-in tiles both, beside MIOpen ("conv1x1_sweep")
   --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
                      socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
@@ -45,12 +39,74 @@ HBM_PEAK_GBS = 8000.0
 PRE_ROLL = 40                                            # untimed launches that bring the part out of idle clocks
 NOMINAL_SCLK_MHZ = 2400.0
 
-# L2<->fabric bytes per launch of the headline kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
-# (KiB per dispatch), each scaled by what the same counter reads for this file's 2^28-byte calibration pass.
-# The two readings and the two factors are in profiles/gemm_tile_c2_clock_power_counters.md (section 4).
-TRAFFIC_KIB_C2 = {"fetch": 788937.5, "fetch_scale": 2.0, "write": 187422.1, "write_scale": 1.0}
-TRAFFIC_BYTES_C2 = int((TRAFFIC_KIB_C2["fetch"] * TRAFFIC_KIB_C2["fetch_scale"]
-                        + TRAFFIC_KIB_C2["write"] * TRAFFIC_KIB_C2["write_scale"]) * 1024)
+# L2<->fabric bytes per launch of the headline kernel come from two `rocprofv3 --pmc` runs of this file (FETCH_SIZE,
+# then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 2^28-byte calibration pass
+# below.  The readings live in profiles/c2_hbm_traffic.json together with the SHA-256 of the kernel sources they were
+# taken from; a record taken from other sources is stale and is not reported.
+TRAFFIC_RECORD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "c2_hbm_traffic.json")
+KERNEL_SOURCES = ("tritonix_amd/csrc/gemm_tile.h", "tritonix_amd/csrc/capi.hip", "tritonix_amd/csrc/registry.h")
+
+
+def kernel_source_hash():
+    """SHA-256 over the sources the tile kernels and their launch code are built from."""
+    import hashlib
+
+    h = hashlib.sha256()
+    root = os.path.dirname(os.path.abspath(__file__))
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(root, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def recorded_traffic(tile):
+    """(bytes per launch, note) from the counter record, or (None, why) when the record does not describe this build."""
+    try:
+        with open(TRAFFIC_RECORD) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter record (profiles/c2_hbm_traffic.json)"
+    if rec.get("kernel_source_sha256") != kernel_source_hash():
+        return None, "counter record is from other kernel sources: re-run the two --pmc passes named in it"
+    if rec.get("tile") != tile:
+        return None, "counter record is for another tile configuration"
+    nbytes = int((rec["fetch_kib"] * rec["fetch_scale"] + rec["write_kib"] * rec["write_scale"]) * 1024)
+    return nbytes, "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/c2_hbm_traffic.json"
+
+
+def write_traffic_record(fetch_csv, write_csv, tile):
+    """Build profiles/c2_hbm_traffic.json from the counter_collection.csv files of
+        rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d DIR -o p -- python3 bench.py --only C2 --no-cpu --no-vendor
+    and the same with WRITE_SIZE.  Each reading (KiB per dispatch, mean over the headline kernel's dispatches) is kept
+    with the factor that makes the same counter read 2^28 bytes for the calibration pass of main()."""
+    import csv
+
+    def reading(path, counter):
+        cal, kern = [], []
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                if "CUDAFunctorOnSelf_add<int>" in row["Kernel_Name"] and int(row["Grid_Size"]) == 1 << 24:
+                    cal.append(float(row["Counter_Value"]))
+                elif "gemm_tile_kernel<tnx::TagBF16" in row["Kernel_Name"]:
+                    kern.append(float(row["Counter_Value"]))
+        if not cal or not kern:
+            raise SystemExit(f"{path}: no {counter} rows for the calibration pass or the headline kernel")
+        return sum(kern) / len(kern), (1 << 28) / 1024.0 / (sum(cal) / len(cal)), len(kern)
+
+    fetch, fetch_scale, n_f = reading(fetch_csv, "FETCH_SIZE")
+    write, write_scale, n_w = reading(write_csv, "WRITE_SIZE")
+    rec = {"kernel_source_sha256": kernel_source_hash(), "kernel_sources": list(KERNEL_SOURCES), "tile": tile,
+           "fetch_kib": round(fetch, 1), "fetch_scale": round(fetch_scale, 3), "write_kib": round(write, 1),
+           "write_scale": round(write_scale, 3), "dispatches": [n_f, n_w],
+           "bytes_per_launch": int((fetch * round(fetch_scale, 3) + write * round(write_scale, 3)) * 1024),
+           "algorithmic_bytes": 3 * 8192 * 8192 * 2}
+    with open(TRAFFIC_RECORD, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    return rec
+
 
 ALL = ("C2", "C1", "C3", "C4", "C5", "FFN", "CONV")
 
@@ -65,17 +121,12 @@ def parse():
     ap.add_argument("--operands", choices=("random", "zeros"), default="random")
     ap.add_argument("--splitk-reduce", choices=("ordered", "atomic"), default="ordered",
                     help="C3 only: how the K slices meet (ordered = stored apart, summed in slice order; atomic = fp32 atomic adds)")
-    ap.add_argument("--mfma-ceiling", action="store_true",
-                    help="also time the MFMA-only loop (no data movement) for both MFMA shapes and both operand kinds")
-    ap.add_argument("--shape-sweep", action="store_true",
-                    help="also time the built-in tile choice on a ladder of other bf16 shapes (GEMV to 2048^3, aligned "
-                         "and ragged) beside the vendor library's GEMM on the same operands (\"shape_sweep\")")
-    ap.add_argument("--conv1x1-sweep", action="store_true",
-                    help="also time ResNet-50's 1x1 layers on the GEMM route and on the conv2d kernels (\"conv1x1_sweep\")")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocBLAS/hipBLASLt timing of the same operands")
+    ap.add_argument("--traffic-from", default=None, metavar="FETCH_CSV,WRITE_CSV",
+                    help="no GPU: write profiles/c2_hbm_traffic.json from the counter_collection.csv files of two rocprofv3 --pmc runs")
     ap.add_argument("--tile", default=None, help="headline tile override: block_m,block_n,block_k,num_warps,num_stages,group_m")
     return ap.parse_args()
 
@@ -208,132 +259,20 @@ def sustain(step, seconds, flops):
     return out
 
 
-SWEEP_SHAPES = [(1, 4096, 4096), (8, 14336, 4096), (32, 4096, 14336), (64, 8192, 8192), (128, 8192, 8192),
-                (512, 4096, 4096), (1024, 1024, 1024), (2048, 2048, 512), (2048, 2048, 2048), (1024, 4096, 4096),
-                (3072, 3072, 3072), (4096, 4096, 4096),
-                (4096, 4096, 4104), (4096, 4100, 4096), (4100, 4096, 4096),
-                (512, 4096, 4096, "kc"), (4096, 4096, 4096, "kc"), (4096, 14336, 4096, "kc"), (8192, 8192, 8192, "kc")]
-
-
-def shape_sweep(torch, dev, mm):
-    """Kernel time of the built-in configuration (`tnx_gemm_default_config`) on other shapes, launches bound once
-    (`prepare`), B rotated over several copies so that skinny shapes stream it from HBM; the vendor's GEMM on the
-    same operands beside it."""
-    rows = []
-    for m, n, k, *layout in SWEEP_SHAPES:
-        g = torch.Generator("cpu").manual_seed(m + n + k)
-        a = (torch.randn(m, k, generator=g) / k ** 0.5).bfloat16().to(dev)
-        if layout:      # "kc": B is the transposed view of an [n, k] weight, the `x @ w.t()` of a linear layer
-            b0 = torch.randn(n, k, generator=g).bfloat16()
-            bs = [b0.to(dev).clone().t() for _ in range(4 if k * n * 2 < 300e6 else 2)]
-        else:
-            b0 = torch.randn(k, n, generator=g).bfloat16()
-            bs = [b0.to(dev).clone() for _ in range(4 if k * n * 2 < 300e6 else 2)]
-        cfg = mm.default_config(a, bs[0])
-        kern = mm.gemm_splitk_kernel if cfg.get("split_k", 1) > 1 else mm.matmul_kernel
-        c = torch.empty((m, n), device=dev, dtype=torch.bfloat16)
-        ls = [kern.prepare(a, b, c, m, n, k, a.stride(0), 1, b.stride(0), b.stride(1), n, 1, **cfg) for b in bs]
-        pre_roll(lambda i: ls[i % len(ls)]())
-        ours = region_time(lambda i: ls[i % len(ls)](), 50)
-        pre_roll(lambda i: torch.matmul(a, bs[i % len(bs)], out=c))
-        vendor = region_time(lambda i: torch.matmul(a, bs[i % len(bs)], out=c), 50)
-        rows.append({"shape": [m, n, k], "b_layout": "k-contiguous" if layout else "row-major", "ms": round(ours, 4), "tflops": round(2.0 * m * n * k / ours / 1e9, 1),
-                     "gbs": round(2.0 * (m * k + k * n + m * n) / ours / 1e6, 1), "vendor_ms": round(vendor, 4),
-                     "config": cfg})
-    return rows
-
-
-# c_in, plane side, c_out of the 1x1 layers of a ResNet-50 (unit stride: the projections inside the bottleneck blocks)
-CONV1X1_LAYERS = [(64, 56, 256), (256, 56, 64), (256, 56, 128), (256, 56, 512), (512, 28, 128), (128, 28, 512),
-                  (512, 28, 1024), (1024, 14, 256), (256, 14, 1024), (1024, 14, 2048), (2048, 7, 512), (512, 7, 2048)]
-
-
-def conv1x1_sweep(torch, dev):
-    """Kernel time of the 1x1 layers with the library's own tile: the GEMM route (LOADER="gemm"), the conv2d kernel
-    "auto" would take without that route (direct-to-LDS where it applies, else register-staged), what "auto" takes,
-    and the vendor's conv2d on the same tensors.  Launches bound once (`prepare`)."""
-    import ctypes
-
-    from tritonix_amd import _C
-    from tritonix_amd.ops.conv2d import forward as conv
-
-    rows = []
-    zero = dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0, GROUP_SIZE_M=8)
-    for batch in (8, 32, 128):
-        for c_in, hw, c_out in CONV1X1_LAYERS:
-            g = torch.Generator("cpu").manual_seed(batch + c_in + hw)
-            x = torch.randn(batch, c_in, hw, hw, generator=g).bfloat16().to(dev)
-            w = (torch.randn(c_out, c_in, 1, 1, generator=g) / c_in ** 0.5).bfloat16().to(dev)
-            bias = torch.randn(c_out, generator=g).bfloat16().to(dev)
-            y = torch.empty(batch, c_out, hw, hw, device=dev, dtype=torch.bfloat16)
-
-            def bound(loader):
-                return conv.conv2d_forward_kernel.prepare(y, x, w, bias, batch, c_in, hw, hw, c_out, hw, hw, 1, 1, 1, 1, 0, 0,
-                                                          1, 1, batch * hw * hw, c_out, c_in, LOADER=loader, **zero)
-
-            def timed(fn):
-                pre_roll(lambda i: fn())
-                return region_time(lambda i: fn(), 50)
-
-            other, other_name = bound("dma"), "dma"
-            if _C.load().tnx_conv2d_supported(ctypes.byref(other.args)) != _C.OK:
-                other, other_name = bound("registers"), "registers"
-            auto = bound("auto")
-            row = {"batch": batch, "layer": [c_in, hw, c_out], "gemm_us": round(timed(bound("gemm")) * 1e3, 1),
-                   "conv2d_us": round(timed(other) * 1e3, 1), "conv2d_kernel": other_name,
-                   "auto_us": round(timed(auto) * 1e3, 1), "auto_takes": {1: "registers", 2: "dma", 3: "gemm"}[builtin_loader(auto.args)],
-                   "vendor_us": round(timed(lambda: torch.nn.functional.conv2d(x, w, bias)) * 1e3, 1)}
-            row["gbs_auto"] = round(2.0 * (x.numel() + w.numel() + y.numel()) / row["auto_us"] / 1e3, 1)
-            rows.append(row)
-    return rows
-
-
-def builtin_loader(conv_args):
-    """The loader `tnx_conv2d_default_config` names for this problem (tnx_conv_loader)."""
-    import ctypes
-
-    from tritonix_amd import _C
-
-    probe = type(conv_args).from_buffer_copy(conv_args)
-    st = _C.load().tnx_conv2d_default_config(ctypes.byref(probe))
-    assert st == _C.OK, _C.strerror(st)
-    return probe.loader
-
-
-def mfma_ceiling(torch, dev, dtype_code, peak):
-    """T(FL)OP/s of the MFMA-only loop: {"16x16": {"random": .., "zeros": ..}, "32x32": {...}} (same protocol as the
-    kernels: pre-roll, then one HIP-event pair around back-to-back launches on the launch stream)."""
-    import ctypes
-
-    from tritonix_amd import _C
-
-    lib = _C.load()
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    scratch = torch.empty(cus * 256, dtype=torch.float32, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-    ops = ctypes.c_double()
-    out = {}
-    for rows in (16, 32):
-        for kind, zero in (("random", 0), ("zeros", 1)):
-            def launch(_i=0):
-                st = lib.tnx_probe_mfma(dtype_code, rows, zero, cus, 2000, scratch.data_ptr(), scratch.numel() * 4, stream,
-                                        ctypes.byref(ops))
-                assert st == _C.OK, _C.strerror(st)
-            for _ in range(30):
-                launch()
-            torch.cuda.synchronize()
-            ms = region_time(launch, 40)
-            out.setdefault(f"{rows}x{rows}", {})[kind] = round(ops.value / ms / 1e9, 1)
-    out["peak"] = peak
-    out["frac_of_peak_random_16x16"] = round(out["16x16"]["random"] / peak, 4)
-    return out
-
-
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
+    if args.traffic_from:
+        sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+        mm = __import__("importlib").import_module("tritonix_amd.ops.matmul")
+        import torch
+
+        tile = mm.default_config(torch.empty(8192, 8192, dtype=torch.bfloat16, device="meta"),
+                                 torch.empty(8192, 8192, dtype=torch.bfloat16, device="meta"))
+        print(json.dumps(write_traffic_record(*args.traffic_from.split(","), tile)))
+        return 0
     import torch
 
     if not torch.cuda.is_available():
@@ -386,13 +325,6 @@ def main():
     ok = True
     if "C2" in only:
         ok = headline(torch, dev, oracle, mm, args, operands, out)
-    if args.mfma_ceiling:
-        out["mfma_ceiling"] = {"bf16": mfma_ceiling(torch, dev, _C.BF16, PEAK["bf16"]),
-                               "i8": mfma_ceiling(torch, dev, _C.I8, PEAK["i8"])}
-    if args.shape_sweep:
-        out["shape_sweep"] = shape_sweep(torch, dev, mm)
-    if args.conv1x1_sweep:
-        out["conv1x1_sweep"] = conv1x1_sweep(torch, dev)
     extras_wanted = [s for s in only if s != "C2"]
     if extras_wanted:
         out["per_config"] = extras(torch, dev, oracle, mm, sg, args, operands, extras_wanted)
@@ -436,8 +368,9 @@ def headline(torch, dev, oracle, mm, args, operands, out):
     durs = event_times(step, nev)                    # one event pair per launch: spread of single launches
     kern_ms = region_time(step, nev)                 # one event pair around the region: mean launch duration
     achieved = flops / kern_ms / 1e9
+    traffic, traffic_note = recorded_traffic(cfg) if args.operands == "random" else (None, "not recorded for all-zero operands")
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK["bf16"], "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK["bf16"], 4), "traffic": TRAFFIC_BYTES_C2,
+                "frac": round(achieved / PEAK["bf16"], 4), "traffic": traffic, "traffic_source": traffic_note,
                 "kernel_ms": round(kern_ms, 4), "kernel_ms_single_mean": round(sum(durs) / len(durs), 4),
                 "kernel_ms_single_min": round(min(durs), 4)}
 
@@ -654,6 +587,26 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
             rows = torch.arange(0, 4096, 585)
             hidden = oracle.reference_glu(x_cpu[rows], w_cpu, "silu").bfloat16().float()
             r["parity_ok"] = bool(oracle.within_tolerance(y[rows.to(dev)], hidden @ w3_cpu.float())[0])
+            # What a one-kernel fusion over the intermediate's columns has to move: every column tile of the gated
+            # product (112 of them at this size) contributes a partial [rows, 4096] fp32 sum of the down-projection
+            # that has to meet the others' -- the reference's draft adds them with atomics (tritonix/ops/swiglu.py:
+            # 207-230).  Timed here with this library's own hand-over for K slices: the down-projection alone, K cut 56
+            # ways (half the slices the fusion needs; 3.7 GB of partial sums, the most a 32-bit slice offset
+            # addresses), against the same product uncut.
+            cfg_cut = {"block_m": 256, "block_n": 256, "block_k": 64, "group_m": 8, "num_stages": 2, "num_warps": 4}
+            try:
+                cut = mm.matmul_kernel.prepare(z, w3, y, 4096, 4096, 14336, 14336, 1, 4096, 1, 4096, 1, split_k=56, **cfg_cut)
+                pre_roll(lambda i: cut())
+                t_cut = region_time(lambda i: cut(), 10)
+                pre_roll(lambda i: down())
+                t_down = region_time(lambda i: down(), 20)
+                r["fused_partial_sums"] = {"down_projection_uncut_ms": round(t_down, 4), "down_projection_k_cut_56_ms": round(t_cut, 4),
+                                           "partial_sum_bytes": 56 * 4096 * 4096 * 4,
+                                           "note": "half the partial-sum hand-over of a fusion over 112 column tiles, and already longer than "
+                                                   "the whole two-launch block"}
+                del cut
+            except (ValueError, RuntimeError) as e:
+                r["fused_partial_sums"] = {"error": str(e)}
             del w3, y
         del x, w, z
 

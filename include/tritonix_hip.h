@@ -40,7 +40,9 @@ enum tnx_dtype {
   TNX_BF16 = 1, /* bfloat16 */
   TNX_I8 = 2,   /* signed 8-bit */
   TNX_I32 = 3,  /* signed 32-bit (output of the int8 path) */
-  TNX_F32 = 4   /* binary32: the type of split-K slices in the workspace; no entry point takes or returns it */
+  TNX_F32 = 4   /* binary32: the type of split-K slices in the workspace, and an output type: a bf16 / f16 GEMM on
+                   a tile of at most 128x128 may write its fp32 sums unrounded (out_dtype = TNX_F32).  No kernel
+                   takes binary32 operands; tnx_split_f32 turns them into bf16 operands of a three-term product */
 };
 
 /* epilogues fused after the K loop (tritonix/ops/swiglu.py:98-104).
@@ -181,30 +183,24 @@ int tnx_gemm_default_config(tnx_gemm_args* args);
  * TNX_SCHED_SUPERBLOCK: the super-block order.  Either is a bijection of [0, tiles_m*tiles_n) onto the grid. */
 int tnx_tile_coords(int schedule, int id, int tiles_m, int tiles_n, int group_m, int* tile_m, int* tile_n);
 
+/* float32 operands.  The reference's kernels take whatever tl.dot takes (tritonix/ops/matmul.py:98), float32 included,
+ * which Triton multiplies in TF32 (`use_tf32`, tritonix/ops/swiglu.py:89-93).  gfx950 has no TF32 matrix instruction;
+ * a float32 product runs here on the bf16 instructions as three terms: with x = hi(x) + lo(x) + O(2^-17 |x|), hi and lo
+ * both bf16 (round to nearest even), a @ b = hi(a) @ hi(b) + hi(a) @ lo(b) + lo(a) @ hi(b) + O(2^-16), accumulated
+ * in fp32 -- tighter than TF32's 2^-11.  tnx_split_f32 writes the bf16 operand of that product for one float32
+ * matrix src[rows, cols] (element strides stride_r, stride_c), contiguous and row-major in dst:
+ *   side 0 (the A operand):  dst[rows, 3 * cols] = [ hi | hi | lo ]      side 1 (the B operand):  dst[3 * rows, cols] = [ hi ; lo ; hi ]
+ * so that one tnx_gemm with k' = 3k, in_dtype = TNX_BF16 and out_dtype = TNX_F32 (or a GLU epilogue on top) is the
+ * float32 product.  Non-finite elements keep their head and get a zero tail.  dst holds 3 * rows * cols bf16 values.
+ * Asynchronous on `stream`; allocates nothing. */
+int tnx_split_f32(const float* src, int64_t rows, int64_t cols, int64_t stride_r, int64_t stride_c, void* dst, int side,
+                  void* stream);
+
 /* Number of compiled tile kernels, and a description of the i-th one:
  * "dtype bm bn bk warps stages [generic] [persistent]" as a NUL-terminated string (static storage);
  * "generic": also built with the element-wise loader; "persistent": also built for TNX_SCHED_PERSISTENT. */
 int tnx_kernel_count(void);
 const char* tnx_kernel_name(int i);
-
-/* Measurement aid with no counterpart in the reference: launch a kernel of `workgroups` x 4 waves that issues
- * nothing but MFMAs of `dtype` (TNX_F16 / TNX_BF16 / TNX_I8) on operands held in registers -- 16x16 (mfma_rows =
- * 16) or 32x32 (32) tiles, `iterations` x 64 (resp. 32) instructions per wave, operands random (data-like
- * switching activity) or all zero.  The rate it reaches is what the MFMA pipes sustain on this board before any
- * operand has been moved: with random operands it is set by the board's power limit and bounds every GEMM kernel
- * from above.  `scratch` receives workgroups * 1024 bytes of don't-care output; *ops_per_launch (may be NULL) the
- * multiply-add count x 2.  Asynchronous on `stream`; timing is the caller's. */
-int tnx_probe_mfma(int dtype, int mfma_rows, int zero_operands, int workgroups, int iterations, void* scratch,
-                   size_t scratch_bytes, void* stream, double* ops_per_launch);
-
-/* Measurement aid with no counterpart in the reference: one wave issues `iterations` x 8 LDS instructions of one
- * kind, lane l at byte offset lane_offsets[l] (+ u * 4096, u = 0..7) of a 64 KiB LDS array.  lane_offsets is a HOST
- * array of 64 offsets, each at most 32768 and aligned to the access (16 bytes for the b128 forms, 8 for the
- * transposing reads).  Run under `rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_INSTS_LDS`: the
- * conflict cycles per instruction of that address pattern.  `scratch`: 512 bytes of device memory (table and
- * don't-care output).  Asynchronous on `stream` after a 256-byte host-to-device copy. */
-enum tnx_lds_op { TNX_LDS_READ_B128 = 0, TNX_LDS_WRITE_B128 = 1, TNX_LDS_READ_TR16_B64 = 2, TNX_LDS_READ_TR8_B64 = 3 };
-int tnx_probe_lds(int op, const uint32_t* lane_offsets, int iterations, void* scratch, size_t scratch_bytes, void* stream);
 
 /* ---- conv2d forward (implicit GEMM on the same LDS layout and MFMA fragments) ------------------------------
  * Stands in for conv2d_forward_kernel, tritonix/ops/conv2d/forward.py:19-165: contiguous NCHW input, KCRS

@@ -187,20 +187,3 @@ def test_default_config_of_the_benchmark_shapes():
     assert picked == [_C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, _C.SCHED_SUPERBLOCK, 0, 0, 0, _C.SCHED_SUPERBLOCK]
 
 
-def test_lds_probe_rejects_bad_arguments_before_touching_the_gpu():
-    lib = _C.load()
-    ok = (ctypes.c_uint32 * 64)(*[16 * l for l in range(64)])
-    scratch = ctypes.c_void_p(0x1000)                              # never dereferenced: every call below fails on the host
-    assert lib.tnx_probe_lds(7, ok, 10, scratch, 512, None) == _C.E_INVALID          # unknown instruction kind
-    assert lib.tnx_probe_lds(_C.LDS_READ_B128, ok, 0, scratch, 512, None) == _C.E_INVALID
-    assert lib.tnx_probe_lds(_C.LDS_READ_B128, ok, 10, None, 512, None) == _C.E_INVALID
-    assert lib.tnx_probe_lds(_C.LDS_READ_B128, ok, 10, scratch, 256, None) == _C.E_WORKSPACE
-    misaligned = (ctypes.c_uint32 * 64)(*[8 * l for l in range(64)])
-    assert lib.tnx_probe_lds(_C.LDS_READ_B128, misaligned, 10, scratch, 512, None) == _C.E_INVALID
-    beyond = (ctypes.c_uint32 * 64)(*([0] * 63 + [32768 + 16]))
-    assert lib.tnx_probe_lds(_C.LDS_READ_TR16_B64, beyond, 10, scratch, 512, None) == _C.E_INVALID
-    # the pattern generator of the probe script: every offset it would hand over is in range and aligned
-    from tritonix_amd import lds_probe
-    for name, op, offs in lds_probe.patterns():
-        assert len(offs) == 64 and max(offs) <= 32768, name
-        assert all(o % (16 if op in (_C.LDS_READ_B128, _C.LDS_WRITE_B128) else 8) == 0 for o in offs), name

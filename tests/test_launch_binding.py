@@ -113,3 +113,83 @@ def test_new_kernel_objects_follow_the_same_protocol():
     with pytest.raises(ValueError):
         k[(1,)](a, b, c, 256, 384, 512, 512, 1, 384, 1, 384, 1, **TILE)
     assert seen == []                                                   # hooks run only for launches that can happen
+
+
+def test_swiglu_kernel_keeps_the_reference_signature():
+    """``swiglu_kernel[grid](x, w12, w3, z, m, n, k, f, 8 strides, block_m=, block_n=, block_k=, group_m=, block_l=,
+    use_tf32=, activation=)`` (tritonix/ops/swiglu.py:127-152), exported as the reference exports it
+    (tritonix/__init__.py:15)."""
+    from tritonix.ops.swiglu import glu_kernel, swiglu_kernel                                # noqa: F401
+    import tritonix
+
+    assert tritonix.swiglu_kernel is tritonix_amd.swiglu_kernel is swiglu_kernel
+    assert isinstance(swiglu_kernel, tritonix_amd.TunableKernel)
+    assert swiglu_kernel.arg_names[:16] == ["x", "w12", "w3", "z", "m", "n", "k", "f", "stride_xm", "stride_xk", "stride_wk",
+                                            "stride_wn", "stride_w3n", "stride_w3l", "stride_zm", "stride_zl"]
+    assert swiglu_kernel.arg_names[16:23] == ["block_m", "block_n", "block_k", "group_m", "block_l", "use_tf32", "activation"]
+    assert swiglu_kernel.keys == ["m", "n", "k"] and swiglu_kernel.specialize_keys == ["m", "n", "k"]
+    assert list(swiglu_kernel.space) == ["block_m", "block_n", "block_k", "block_l", "group_m", "num_stages", "num_warps"]
+    assert {"block_m", "block_n", "block_k", "block_l", "num_stages"} <= swiglu_kernel.memory_params
+    x, w12, w3 = torch.zeros(128, 256, dtype=torch.bfloat16), torch.zeros(256, 512, dtype=torch.bfloat16), torch.zeros(256, 192, dtype=torch.bfloat16)
+    z = torch.zeros(128, 192, dtype=torch.bfloat16)
+    pos = (x, w12, w3, z, 128, 512, 256, 192, 256, 1, 512, 1, 192, 1, 192, 1)
+    tile = dict(block_m=128, block_n=128, block_k=64, group_m=8, block_l=64, num_stages=2, num_warps=4)
+    bound = swiglu_kernel._bind(pos, dict(tile, activation="sigmoid"))
+    assert bound["f"] == 192 and bound["stride_w3n"] == 192 and bound["block_l"] == 64 and bound["activation"] == "sigmoid"
+    with pytest.raises(TypeError, match="missing"):
+        swiglu_kernel._bind(pos, dict(block_m=128))
+    with pytest.raises(TypeError, match="unexpected"):
+        swiglu_kernel._bind(pos, dict(tile, num_ctas=1))
+    with pytest.raises(ValueError, match="HIP device"):                  # no CPU path here either
+        swiglu_kernel[(1, 4)](*pos, **tile)
+
+
+def test_workspace_handed_out_under_graph_capture_is_never_released(monkeypatch):
+    """A captured launch bakes its split-K workspace pointer into the graph: neither the LRU eviction nor a later,
+    larger request may free that buffer (bookkeeping only; no GPU)."""
+    from tritonix_amd import kernel
+
+    dev = torch.device("cpu", 0)
+    monkeypatch.setattr(kernel, "_workspaces", type(kernel._workspaces)())
+    monkeypatch.setattr(kernel, "_captured_workspaces", [])
+    monkeypatch.setattr(kernel, "_capturing", lambda: True)
+    captured = kernel._workspace(dev, 1, 1 << 20)
+    assert kernel._workspace(dev, 1, 1 << 20) is captured and len(kernel._captured_workspaces) == 1
+    monkeypatch.setattr(kernel, "_capturing", lambda: False)
+    grown = kernel._workspace(dev, 1, 4 << 20)                           # a later launch needs more: a new buffer
+    assert grown is not captured and grown.numel() >= 4 << 20
+    for stream in range(2, 2 + 2 * kernel._MAX_WORKSPACES):                # ... and many other streams push it out of the LRU
+        kernel._workspace(dev, stream, 16)
+    assert len(kernel._workspaces) == kernel._MAX_WORKSPACES
+    assert any(kept is captured for kept in kernel._captured_workspaces)  # still alive for the graph's replays
+
+
+def test_float32_calls_are_rewritten_as_a_three_term_bf16_product():
+    """float32 operands (the reference multiplies them in TF32, tritonix/ops/matmul.py:98) become a bf16 problem with
+    k' = 3k and an fp32 result on a tile of at most 128x128; no kernel takes float32 itself."""
+    from tritonix_amd.ops.matmul import default_config
+
+    a, b = torch.zeros(300, 200), torch.zeros(200, 520)
+    cfg = default_config(a, b)
+    assert cfg["block_m"] * cfg["block_n"] <= 128 * 128
+    g = _C.GemmArgs()
+    g.m, g.n, g.k = 300, 520, 600
+    g.stride_am, g.stride_ak, g.stride_bk, g.stride_bn, g.stride_cm, g.stride_cn = 600, 1, 520, 1, 520, 1
+    g.in_dtype, g.out_dtype = _C.BF16, _C.F32
+    g.block_m, g.block_n, g.block_k, g.group_m, g.num_stages, g.num_warps = 128, 128, 64, 8, 3, 8
+    g.split_k = 1
+    lib = _C.load()
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK
+    g.epilogue = _C.EPI_GLU_SILU
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK                # the gated epilogue writes fp32 too
+    g.epilogue = _C.EPI_NONE
+    g.block_m, g.block_n, g.num_stages, g.num_warps = 256, 256, 2, 4       # no fp32 epilogue in the large tiles
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.E_UNSUPPORTED
+    g.block_m, g.block_n, g.block_k, g.num_stages, g.num_warps = 128, 128, 128, 2, 4
+    g.in_dtype = _C.I8
+    assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.E_UNSUPPORTED     # int8 accumulates into int32 only
+    # argument checks of the splitter run on the host
+    assert lib.tnx_split_f32(None, 4, 4, 4, 1, None, 0, None) == _C.E_INVALID
+    assert lib.tnx_split_f32(None, 0, 4, 4, 1, None, 0, None) == _C.OK     # nothing to do
+    assert lib.tnx_split_f32(None, 4, 4, 4, 1, None, 2, None) == _C.E_INVALID
+    assert lib.tnx_split_f32(None, -1, 4, 4, 1, None, 0, None) == _C.E_INVALID

@@ -25,13 +25,11 @@ SCHED_DEFAULT, SCHED_PERSISTENT, SCHED_SUPERBLOCK, SCHED_ATOMIC_REDUCE = 0, 1, 2
 # enum tnx_status
 OK, E_INVALID, E_UNSUPPORTED, E_LDS, E_WORKSPACE, E_HIP, E_STATIC_LIMIT = 0, 1, 2, 3, 4, 5, 6
 STATIC_WORKSPACE_BYTES = 65536 + (32 << 20)
-# enum tnx_lds_op
-LDS_READ_B128, LDS_WRITE_B128, LDS_READ_TR16_B64, LDS_READ_TR8_B64 = 0, 1, 2, 3
 # enum tnx_conv_loader
 CONV_LOADER_AUTO, CONV_LOADER_REGISTERS, CONV_LOADER_DMA, CONV_LOADER_GEMM = 0, 1, 2, 3
 
 EXPORTS = ("tnx_gemm", "tnx_gemm_static_workspace", "tnx_gemm_workspace_bytes", "tnx_gemm_lds_bytes", "tnx_gemm_supported",
-           "tnx_gemm_default_config", "tnx_tile_coords", "tnx_probe_mfma", "tnx_probe_lds", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
+           "tnx_gemm_default_config", "tnx_tile_coords", "tnx_split_f32", "tnx_kernel_count", "tnx_kernel_name", "tnx_strerror",
            "tnx_last_hip_error", "tnx_version", "tnx_conv2d_forward", "tnx_conv2d_supported", "tnx_conv2d_output_size",
            "tnx_conv2d_default_config", "tnx_conv2d_kernel_count", "tnx_conv2d_kernel_name")
 
@@ -96,12 +94,9 @@ def load() -> ctypes.CDLL:
     lib.tnx_gemm_default_config.restype = ctypes.c_int
     lib.tnx_tile_coords.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_int)] * 2
     lib.tnx_tile_coords.restype = ctypes.c_int
-    lib.tnx_probe_mfma.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
-                                                        ctypes.POINTER(ctypes.c_double)]
-    lib.tnx_probe_mfma.restype = ctypes.c_int
-    lib.tnx_probe_lds.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_uint32), ctypes.c_int, ctypes.c_void_p,
-                                  ctypes.c_size_t, ctypes.c_void_p]
-    lib.tnx_probe_lds.restype = ctypes.c_int
+    lib.tnx_split_f32.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                  ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    lib.tnx_split_f32.restype = ctypes.c_int
     lib.tnx_kernel_count.argtypes = []
     lib.tnx_kernel_count.restype = ctypes.c_int
     lib.tnx_kernel_name.argtypes = [ctypes.c_int]

@@ -11,7 +11,10 @@ from __future__ import annotations
 
 import argparse
 import concurrent.futures as cf
+import glob
+import json
 import os
+import re
 import subprocess
 import sys
 import time
@@ -233,6 +236,47 @@ def generate(instances):
     return files
 
 
+# A compiler-generated use of M0 would collide with the DMA loader: its inline assembly writes M0 (the LDS target of
+# global_load_lds) and cannot name it as clobbered.  Every device translation unit is therefore compiled with its
+# assembly kept, and any mention of m0 outside an inline-assembly block fails the build.
+_M0 = re.compile(r"(?<![\w.$])m0(?![\w])")
+_REMARK = re.compile(r"remark: .*?:\d+:\d+:\s+(Function Name|TotalSGPRs|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|Occupancy \[waves/SIMD\]|"
+                     r"SGPRs Spill|VGPRs Spill|LDS Size \[bytes/block\]): (\S+)")
+
+
+def compiler_m0_uses(asm_path):
+    """(line number, text) of every instruction outside inline assembly that names M0."""
+    found, inside = [], False
+    with open(asm_path, errors="replace") as f:
+        for n, line in enumerate(f, 1):
+            if ";;#ASMSTART" in line:
+                inside = True
+            elif ";;#ASMEND" in line:
+                inside = False
+            elif not inside and _M0.search(line.split(";", 1)[0]):
+                found.append((n, line.strip()))
+    return found
+
+
+def parse_resources(stderr):
+    """{mangled kernel name: {"sgpr", "vgpr", "agpr", "scratch", "occupancy", "sgpr_spill", "vgpr_spill", "lds"}} from the
+    compiler's -Rpass-analysis=kernel-resource-usage remarks (no disassembly involved)."""
+    names = {"TotalSGPRs": "sgpr", "VGPRs": "vgpr", "AGPRs": "agpr", "ScratchSize [bytes/lane]": "scratch",
+             "Occupancy [waves/SIMD]": "occupancy", "SGPRs Spill": "sgpr_spill", "VGPRs Spill": "vgpr_spill",
+             "LDS Size [bytes/block]": "lds"}
+    out, cur = {}, None
+    for m in _REMARK.finditer(stderr):
+        key, val = m.group(1), m.group(2)
+        if key == "Function Name":
+            cur = out.setdefault(val, {})
+        elif cur is not None:
+            cur[names[key]] = int(val)
+    return out
+
+
+_resources = {}
+
+
 def _compile(src, obj, verbose, force=True):
     deps = [src, os.path.join(CSRC, "gemm_tile.h"), os.path.join(CSRC, "gemm_skinny.h"), os.path.join(CSRC, "registry.h"),
             os.path.join(CSRC, "conv_tile.h"),
@@ -240,13 +284,32 @@ def _compile(src, obj, verbose, force=True):
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(d) for d in deps):
         return obj
     t0 = time.time()
-    cmd = [HIPCC, *DEVICE_FLAGS, "-c", src, "-o", obj]
+    cmd = [HIPCC, *DEVICE_FLAGS, "-save-temps=obj", "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr[-4000:]}")
+    _resources.update(parse_resources(r.stderr))
+    stem = obj[:-2]
+    asm = f"{stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s"
+    uses = compiler_m0_uses(asm)
+    for tmp in glob.glob(glob.escape(stem) + "-hip-amdgcn-*") + glob.glob(glob.escape(stem) + "-host-*") + glob.glob(glob.escape(stem) + ".hip-hip-*"):
+        os.remove(tmp)
+    if uses:
+        raise RuntimeError(f"{src}: the compiler generated {len(uses)} use(s) of M0 outside inline assembly, e.g. line "
+                           f"{uses[0][0]}: {uses[0][1]} -- the DMA loader's inline assembly owns M0 (gemm_tile.h: dma16)")
     if verbose:
         print(f"  [{time.time() - t0:5.1f}s] {os.path.basename(src)}", flush=True)
     return obj
+
+
+def demangled_tile(name):
+    """'bf16 256x256x64 w4 s2 fast' from a mangled gemm_tile_kernel instantiation (None for other kernels)."""
+    m = re.search(r"gemm_tile_kernelINS_(\d)Tag(\w+?)ENS_7TileCfgIS1_Li(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)EEELb(\d)ELb(\d)ELb(\d)ELb(\d)E", name)
+    if not m:
+        return None
+    _, tag, bm, bn, bk, nw, st, fast, persist, bt, conv = m.groups()
+    kind = "conv" if conv == "1" else "bt" if bt == "1" else "persistent" if persist == "1" else "fast" if fast == "1" else "generic"
+    return f"{tag.lower()} {bm}x{bn}x{bk} w{nw} s{st} {kind}"
 
 
 def build(jobs=None, quick=False, verbose=True, force=True, only=None, out=None, defines=(), only_conv=None):
@@ -263,7 +326,7 @@ def build(jobs=None, quick=False, verbose=True, force=True, only=None, out=None,
         BUILD = os.path.join(ROOT, "build", "dev_" + os.path.basename(lib).replace(".", "_"))
     DEVICE_FLAGS.extend(f"-D{d}" for d in defines)
     srcs = generate(instances) + generate_conv(conv_instances, os.path.join(BUILD, "gen")) + [
-        os.path.join(CSRC, "capi.hip"), os.path.join(CSRC, "skinny.hip"), os.path.join(CSRC, "probe.hip"),
+        os.path.join(CSRC, "capi.hip"), os.path.join(CSRC, "skinny.hip"),
         os.path.join(CSRC, "conv.hip")]
     objdir = os.path.join(BUILD, "obj")
     os.makedirs(objdir, exist_ok=True)
@@ -280,8 +343,13 @@ def build(jobs=None, quick=False, verbose=True, force=True, only=None, out=None,
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     os.replace(lib + ".tmp", lib)
+    # registers, scratch and LDS of every kernel compiled in this run, as the compiler reported them
+    table = {demangled_tile(k) or k: v for k, v in _resources.items()}
+    with open(os.path.join(BUILD, "kernel_resources.json"), "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
     if verbose:
-        print(f"linked {lib} in {time.time() - t0:.1f}s", flush=True)
+        print(f"linked {lib} in {time.time() - t0:.1f}s; no compiler-generated use of M0; "
+              f"kernel resources in {os.path.join(BUILD, 'kernel_resources.json')}", flush=True)
     return lib
 
 

@@ -69,8 +69,13 @@ static int check_common(const tnx_gemm_args* a) {
       a->schedule > (TNX_SCHED_PERSISTENT | TNX_SCHED_SUPERBLOCK | TNX_SCHED_ATOMIC_REDUCE))
     return TNX_E_INVALID;
   // output type is tied to the input type: f16->f16, bf16->bf16, i8->i32
+  // ... or binary32 for the 16-bit float types, on the tiles that carry that epilogue (f32_out_tile in gemm_tile.h)
   int want_out = a->in_dtype == TNX_I8 ? TNX_I32 : a->in_dtype;
-  if (a->out_dtype != want_out) return TNX_E_UNSUPPORTED;
+  if (a->out_dtype != want_out) {
+    const bool f32_out = a->out_dtype == TNX_F32 && a->in_dtype != TNX_I8 && (int64_t)a->block_m * a->block_n <= 128 * 128 &&
+                         !(a->schedule & TNX_SCHED_PERSISTENT) && !is_skinny_cfg(a);
+    if (!f32_out) return TNX_E_UNSUPPORTED;
+  }
   if (a->epilogue != TNX_EPI_NONE && (a->in_dtype == TNX_I8 || (a->n & 1))) return TNX_E_UNSUPPORTED;
   if (a->m > 0x7fffffff || a->n > 0x7fffffff || a->k > 0x7fffffff) return TNX_E_UNSUPPORTED;
   return TNX_OK;
@@ -354,6 +359,16 @@ extern "C" int tnx_gemm_static_workspace(const tnx_gemm_args* a) {
     hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)t.stream, (int*)ptr, words);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+    if (t.schedule & TNX_SCHED_ATOMIC_REDUCE) {
+      // The atomic reduction adds every slice into one copy behind the counters and needs that copy zero at
+      // launch.  A launch of this kind leaves it zero, but the array may hold the slices of an earlier ordered
+      // launch (or of another tile shape), so the copy this launch adds into is cleared first, same fill kernel.
+      const int64_t sum_words = cut_tiles(&t) * (int64_t)t.block_m * t.block_n;   // < 2^23: need <= TNX_STATIC_WORKSPACE_BYTES
+      hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((sum_words + 255) / 256)), dim3(256), 0, (hipStream_t)t.stream,
+                         (int*)((unsigned char*)ptr + WS_COUNTER_BYTES), (int)sum_words);
+      err = hipGetLastError();
+      if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
+    }
     t.workspace = ptr;
     t.workspace_bytes = TNX_STATIC_WORKSPACE_BYTES;
   }
@@ -364,7 +379,13 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   if (!a) return TNX_E_INVALID;
   const int es = elem_size(a->in_dtype);
   const int bk = es == 1 ? 128 : 64;   // 128 bytes of K per LDS row for either element size
-  const int64_t cus = 256;
+  // Workgroups that run together: the CU count of the current device, or MI355X's 256 when no device can be asked
+  // (host-side planning).  The cost constants below are measured on MI355X.
+  int64_t cus = 256;
+  {
+    int n = 0;
+    if (compute_units(&n) == TNX_OK && n > 0) cus = n;
+  }
   a->group_m = 8;
   a->split_k = 1;
   a->tail_tiles = 0;
@@ -414,7 +435,8 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
   const int ncand = 8;
   // int8: rows of a 64-wide B tile are too short for the transposing read; the 192-wide tiles exist for it too
   // (3072 x 4096 x 4096: 53.6 -> 45.7 us with 192x256, 4096 x 3072 x 4096: 52.8 -> 47.3 us with 256x192)
-  auto usable = [&](int i) { return es == 2 || i != 4; };
+  // (a binary32 result exists on the tiles up to 128x128 only)
+  auto usable = [&](int i) { return (es == 2 || i != 4) && (a->out_dtype != TNX_F32 || (i >= 2 && i <= 4)); };
   const double cu_flops = 5.5e12 * (es == 1 ? 1.7 : 1.0);          // per CU with the largest tile
   const double launch = 3e-6, handover = 9e-6, readback = 60e9;
   const int64_t kt = (a->k + bk - 1) / bk;
@@ -467,6 +489,44 @@ extern "C" int tnx_gemm_default_config(tnx_gemm_args* a) {
     const int64_t tm = (a->m + a->block_m - 1) / a->block_m, tn = (a->n + a->block_n - 1) / a->block_n;
     if (bs == 1 && tm >= 16 && tn >= 16) a->schedule = TNX_SCHED_SUPERBLOCK;
   }
+  return TNX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// float32 operands as bf16 head and tail (see tnx_split_f32 in the header)
+// ---------------------------------------------------------------------------
+__global__ void split_f32_kernel(const float* src, int64_t rows, int64_t cols, int64_t sr, int64_t sc, uint16_t* dst, int side) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= rows * cols) return;
+  const int64_t i = idx / cols, j = idx - i * cols;
+  const float v = src[i * sr + j * sc];
+  const __bf16 hi = (__bf16)v;                                        // round to nearest even
+  const float rest = v - (float)hi;
+  const __bf16 lo = (__builtin_isfinite(rest) && __builtin_isfinite(v)) ? (__bf16)rest : (__bf16)0.0f;
+  const uint16_t h = __builtin_bit_cast(uint16_t, hi), l = __builtin_bit_cast(uint16_t, lo);
+  if (side == 0) {
+    uint16_t* row = dst + i * 3 * cols;
+    row[j] = h;
+    row[cols + j] = h;
+    row[2 * cols + j] = l;
+  } else {
+    dst[i * cols + j] = h;
+    dst[(rows + i) * cols + j] = l;
+    dst[(2 * rows + i) * cols + j] = h;
+  }
+}
+
+extern "C" int tnx_split_f32(const float* src, int64_t rows, int64_t cols, int64_t stride_r, int64_t stride_c, void* dst, int side,
+                             void* stream) {
+  if (rows < 0 || cols < 0 || (side != 0 && side != 1)) return TNX_E_INVALID;
+  if (rows == 0 || cols == 0) return TNX_OK;
+  if (!src || !dst) return TNX_E_INVALID;
+  const int64_t total = rows * cols;
+  if (rows > 0x7fffffff || cols > 0x7fffffff || (total + 255) / 256 > 0x7fffffffll) return TNX_E_UNSUPPORTED;
+  hipLaunchKernelGGL(split_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, src, rows, cols,
+                     stride_r, stride_c, (uint16_t*)dst, side);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) { g_last_hip_error = (int)err; return TNX_E_HIP; }
   return TNX_OK;
 }
 

@@ -21,6 +21,16 @@
 #include <type_traits>
 #include <stdint.h>
 
+// Attribution builds (never the shipped library): -D TNX_LADDER=n strips the K loop of the DMA kernels down to a rung
+// of the ladder  1: MFMAs only (both fragment sets filled once from the first slab)  2: + the fragment reads from
+// LDS and the per-slab barrier, no refill of the ring  3: + the refill, but always of the tile's first slabs, so every
+// load is served by the L2  4: the full loop without its waits for the loads  (0: the kernel as shipped).  Results
+// of rungs 1-4 are wrong on purpose; they are timed with power and clock sampling beside the full kernel to say
+// what each part of the loop costs on a power-limited board.
+#ifndef TNX_LADDER
+#define TNX_LADDER 0
+#endif
+
 namespace tnx {
 
 typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -412,6 +422,13 @@ struct OutF16 {
   typedef uint16_t raw;
   static __device__ __forceinline__ raw cvt(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 };
+// binary32 output of a 16-bit-float GEMM: the accumulator as it is.  It is what lets a float32 product run on the
+// bf16 matrix instructions as a three-term split (the host side cuts each operand into a bf16 head and a bf16 tail
+// and lays the terms out along K); built for the tiles up to 128x128 (f32_out_tile).
+struct OutF32 {
+  typedef float raw;
+  static __device__ __forceinline__ raw cvt(float v) { return v; }
+};
 template <class T> struct OutOf;
 template <> struct OutOf<TagBF16> { typedef OutBF16 type; };
 template <> struct OutOf<TagF16> { typedef OutF16 type; };
@@ -439,6 +456,14 @@ template <class O, bool GLU> struct Pack16<O, float, GLU> {   // 16-bit float ou
   static __device__ __forceinline__ void run(const float* f, int epi, raw* out) {
 #pragma unroll
     for (int x = 0; x < OUTV; ++x) out[x] = O::cvt(GLU ? glu_gate(f[2 * x], epi) * f[2 * x + 1] : f[x]);
+  }
+};
+template <bool GLU> struct Pack16<OutF32, float, GLU> {       // binary32 outputs: 4 per lane
+  typedef float raw;
+  static constexpr int OUTV = 4, NF = GLU ? 8 : 4;
+  static __device__ __forceinline__ void run(const float* f, int epi, raw* out) {
+#pragma unroll
+    for (int x = 0; x < OUTV; ++x) out[x] = GLU ? glu_gate(f[2 * x], epi) * f[2 * x + 1] : f[x];
   }
 };
 template <bool GLU> struct Pack16<int, int, GLU> {            // int32 outputs: 4 per lane
@@ -515,6 +540,8 @@ __device__ __forceinline__ void sum_slices(__amdgpu_buffer_rsrc_t win, uint32_t 
 }
 
 template <class C> constexpr bool multi_problem_tile() { return C::BM * C::BN <= 128 * 128; }
+// tiles whose kernels carry a second copy of the epilogue that writes binary32 (16-bit float inputs only)
+template <class T, class C> constexpr bool f32_out_tile() { return T::ES == 2 && C::BM * C::BN <= 128 * 128; }
 
 __device__ __forceinline__ float bias_value(const uint8_t* bias, int row, int dtype) {
   if (dtype == DT_F32) return ((const float*)bias)[row];
@@ -896,6 +923,7 @@ __device__ __forceinline__ void epilogue_store_conv(ACC (&acc)[C::TM][C::TN], ui
   }
 }
 
+template <class X> struct TypeTag { typedef X type; };
 template <bool B> struct BoolTag { static constexpr bool value = B; };
 template <int V> struct IntTag { static constexpr int value = V; };
 
@@ -945,21 +973,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // Phase trace (builds with -DTNX_PHASE_TRACE only; tritonix_amd/phase_trace.py reads it): wave 0 of every
-  // workgroup of the one-tile-per-workgroup kernel leaves the 100 MHz timestamp of its start, of the first slab's
-  // arrival, of its last MFMA and of its last store instruction, and the two hardware-id registers that name its
-  // CU, in 64 bytes of the workspace (uncut launches that are handed a workspace only).  (The branch is on the wave id, not the thread id: a divergent branch here
-  // made the compiler carry the DMA base pointers in vector registers, which the loads cannot take.)
-#ifdef TNX_PHASE_TRACE
-#define TNX_PHASE(i) do { if (wave == 0 && p.ws && p.split_k == 1) ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-  if (wave == 0 && p.ws && p.split_k == 1) {
-    ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + 4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);    // HW_ID
-    ((volatile uint64_t*)p.ws)[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);   // XCC_ID
-  }
-  TNX_PHASE(0);
-#else
-#define TNX_PHASE(i)
-#endif
 
   // ---- which tile / split ------------------------------------------------
   // Tiles [0, split_tile0) in launch order are computed whole by one workgroup each; the
@@ -1414,6 +1427,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     else dma16_go<false>(b_sbase, b_voff[q - C::A_LPW]);
   };
   auto dma_advance = [&]() __attribute__((always_inline)) {
+    if (TNX_LADDER == 3) return;        // + DMA ops, always of the tile's first slabs (served by the L2)
     a_sbase += BK * ES;
     if (!CONV) b_sbase += BT ? (int64_t)BK * ES : (int64_t)BK * p.sbk * ES;
   };
@@ -1517,6 +1531,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   auto slot_body = [&](int mset, int x, int rset, int& rd, uint32_t sa, uint32_t sb, int ks_next, bool with_dma, int slot,
                        uint32_t dst) __attribute__((always_inline)) {
     mma_one(mset, x);
+    if (TNX_LADDER == 1) {              // MFMAs only
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
+    if (TNX_LADDER == 2) with_dma = false;   // + fragment reads: the ring keeps the slabs of the prologue
     if (with_dma) conv_fix_slot(slot);
     int lo = 0, hi = 0;
     if (with_dma && slot < SPAN) { lo = slot * C::LPW / SPAN; hi = (slot + 1) * C::LPW / SPAN; }
@@ -1632,6 +1651,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     const uint32_t sa = stage_of(0), sb = sa + C::A_BYTES;
 #pragma unroll
     for (int r = 0; r < NREAD; ++r) read_one(0, r, sa, sb, 0);
+    if (TNX_LADDER == 1) {
+#pragma unroll
+      for (int r = 0; r < NREAD; ++r) read_one(1, r, sa, sb, C::KSTEPS > 1 ? 1 : 0);
+    }
     inner_steps(sa, sb, No{}, 0u, Par0{});
   }
 
@@ -1648,8 +1671,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       auto period = [&](auto jtag) __attribute__((always_inline)) {
         constexpr int j = decltype(jtag)::value;
         constexpr int P = (C::KSTEPS & 1) ? (j & 1) : 0;          // parity of the slab whose last k step runs now
-        __builtin_amdgcn_s_waitcnt((PWAIT & 0xF) | (((PWAIT >> 4) & 0x3) << 14) | 0x0070);
-        __builtin_amdgcn_s_barrier();
+        if (TNX_LADDER != 1) {
+          if (TNX_LADDER != 4) __builtin_amdgcn_s_waitcnt((PWAIT & 0xF) | (((PWAIT >> 4) & 0x3) << 14) | 0x0070);
+          __builtin_amdgcn_s_barrier();
+        }
         __builtin_amdgcn_sched_barrier(0);
         conv_period_begin();
         const uint32_t dst = lds0 + (uint32_t)(j % STAGES) * C::STAGE_BYTES;
@@ -1718,7 +1743,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       issue_prologue();
       if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
     }
-    TNX_PHASE(1);
     k_loop();
     if constexpr (FAST && !CONV) {
       if (tail_here) {
@@ -1736,7 +1760,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
         }
       }
     }
-    TNX_PHASE(2);
 
     // ---- epilogue ------------------------------------------------------------
     // every wave is done with the slabs before the LDS is reused for the output strips
@@ -1748,31 +1771,41 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
       epilogue_store_conv<T, C, O>(acc, p.c, strip, lane, (int)gm0, (int)gn0, p.cv);
       return;
     }
-    if (cut) {
-      // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
-      const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;
-      const int64_t slice_stride = (int64_t)ncut * BM * BN * 4;
-      uint8_t* wave0 = p.ws + WS_COUNTER_BYTES + ((int64_t)ctile * NW + wave) * (C::WTM * C::WTN * 4);
-      const bool atomic = p.atomic_reduce != 0;
-      if (!splitk_arrive<T, C>(acc, wave0 + (atomic ? 0 : split * slice_stride), strip, lane, gm0, p.m, (int*)p.ws + ctile,
-                               (int*)smem, p.split_k, atomic))
+    // the output type: the input's own 16-bit type (int32 for int8), or binary32 where that epilogue is built
+    auto finish = [&](auto otag) __attribute__((always_inline)) {
+      typedef typename decltype(otag)::type OT;
+      if (cut) {
+        // workspace after the counters: [slice][cut tile][wave][group][lane] 16-byte elements
+        const int ncut = ntiles - p.split_tile0, ctile = logical - p.split_tile0;
+        const int64_t slice_stride = (int64_t)ncut * BM * BN * 4;
+        uint8_t* wave0 = p.ws + WS_COUNTER_BYTES + ((int64_t)ctile * NW + wave) * (C::WTM * C::WTN * 4);
+        const bool atomic = p.atomic_reduce != 0;
+        if (!splitk_arrive<T, C>(acc, wave0 + (atomic ? 0 : split * slice_stride), strip, lane, gm0, p.m, (int*)p.ws + ctile,
+                                 (int*)smem, p.split_k, atomic))
+          return;
+        const SliceSrc src = {wave0, (uint32_t)slice_stride, atomic ? 1 : p.split_k, atomic};
+        if (p.epilogue == EPI_NONE)
+          epilogue_store<T, C, OT, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0);
+        else
+          epilogue_store<T, C, OT, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                               p.c_row_ok, p.epilogue);
+      } else {
+        const SliceSrc none = {nullptr, 0, 0, false};
+        if (p.epilogue == EPI_NONE)
+          epilogue_store<T, C, OT, false, false, MULTI>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0,
+                                                        p.cv.bias, p.cv.bias_dtype);
+        else
+          epilogue_store<T, C, OT, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
+                                                p.c_row_ok, p.epilogue);
+      }
+    };
+    if constexpr (f32_out_tile<T, C>()) {
+      if (p.out_dtype == DT_F32) {
+        finish(TypeTag<OutF32>{});
         return;
-      const SliceSrc src = {wave0, (uint32_t)slice_stride, atomic ? 1 : p.split_k, atomic};
-      if (p.epilogue == EPI_NONE)
-        epilogue_store<T, C, O, false, true>(acc, src, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0);
-      else
-        epilogue_store<T, C, O, true, true>(acc, src, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                            p.c_row_ok, p.epilogue);
-    } else {
-      const SliceSrc none = {nullptr, 0, 0, false};
-      if (p.epilogue == EPI_NONE)
-        epilogue_store<T, C, O, false, false, MULTI>(acc, none, p.c, strip, lane, gm0, gn0, p.m, p.n, p.scm, p.scn, p.c_row_ok, 0,
-                                                     p.cv.bias, p.cv.bias_dtype);
-      else
-        epilogue_store<T, C, O, true, false>(acc, none, p.c, strip, lane, gm0, gn0 >> 1, p.m, p.n >> 1, p.scm, p.scn,
-                                             p.c_row_ok, p.epilogue);
+      }
     }
-    TNX_PHASE(3);
+    finish(TypeTag<O>{});
   } else {
     // ---- persistent: this workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... ------------
     // The host launches it only with KT >= STAGES.  While the epilogue of a tile runs, the first

@@ -97,10 +97,19 @@ template <class T, class C> struct ConvLaunch<T, C, true> {
   static constexpr launch_fn fn = &launch_tile<T, C, true, false, false, true>;
 };
 
+// The element-wise loader is built only for the tiles that ask for it (a conditional expression would instantiate
+// the kernel for every tile and merely not point at it).
+template <class T, class C, bool WANTED> struct GenericLaunch {
+  static constexpr launch_fn fn = nullptr;
+};
+template <class T, class C> struct GenericLaunch<T, C, true> {
+  static constexpr launch_fn fn = &launch_tile<T, C, false>;
+};
+
 #define TNX_ENTRY(TAG, BM, BN, BK, NW, ST, GENERIC)                                                          \
   {TAG::ID, BM, BN, BK, NW, ST, TileCfg<TAG, BM, BN, BK, NW, ST>::LDS_BYTES,                                 \
    &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, true>,                                                \
-   GENERIC ? &launch_tile<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, false> : (launch_fn) nullptr,               \
+   GenericLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>, GENERIC>::fn,                                        \
    PersistLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn, BtLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn,     \
    ConvLaunch<TAG, TileCfg<TAG, BM, BN, BK, NW, ST>>::fn}
 

@@ -39,12 +39,12 @@ def _torch_dtype_code(dtype) -> int:
     table = {torch.float16: _C.F16, torch.bfloat16: _C.BF16, torch.int8: _C.I8, torch.int32: _C.I32,
              torch.float32: _C.F32}
     if dtype not in table:
-        raise ValueError(f"dtype {dtype} has no HIP kernel (float16, bfloat16 and int8 inputs are built)")
+        raise ValueError(f"dtype {dtype} has no HIP kernel (float16, bfloat16, int8 and -- as a bf16 split -- float32 inputs are built)")
     return table[dtype]
 
 
 def out_dtype_for(dtype):
-    """Output dtype of the engine for an input dtype: 16-bit floats keep theirs, int8 accumulates to int32."""
+    """Output dtype of the engine for an input dtype: floats keep theirs, int8 accumulates to int32."""
     import torch
 
     return torch.int32 if dtype == torch.int8 else dtype
@@ -73,15 +73,60 @@ def _workspace(device, stream_ptr: int, nbytes: int, atomic: bool = False):
         buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     _workspaces.move_to_end(key)
+    if _capturing():
+        # A launch recorded into a HIP graph bakes this pointer into the graph: the buffer must outlive every
+        # replay, so it is never released (not by the eviction below, not when a later call needs a larger one).
+        if not any(kept is buf for kept in _captured_workspaces):
+            _captured_workspaces.append(buf)
+        return buf
     while len(_workspaces) > _MAX_WORKSPACES:
         _workspaces.popitem(last=False)       # launches already enqueued keep their buffer alive through the allocator's stream ordering
     return buf
+
+
+# scratch buffers handed to launches that were recorded into a HIP graph: alive until the process ends
+_captured_workspaces: list = []
+
+
+def _capturing() -> bool:
+    import torch
+
+    try:
+        return bool(torch.cuda.is_current_stream_capturing())
+    except (RuntimeError, AssertionError):
+        return False
 
 
 def drop_workspace(device, stream_ptr: int) -> None:
     """Forget the scratch of (device, stream): called when a launch on it reported an error."""
     for atomic in (False, True):
         _workspaces.pop(_workspace_key(device, stream_ptr, atomic), None)
+
+
+def split_f32_operands(bound: dict, stream: int) -> dict:
+    """A bound float32 call rewritten as the bf16 call that computes it.
+
+    The reference's kernels take float32 operands and multiply them in TF32 (tritonix/ops/matmul.py:98,
+    tritonix/ops/swiglu.py:89-93); gfx950 has no TF32 matrix instruction.  ``tnx_split_f32`` cuts each operand into a
+    bf16 head and a bf16 tail and lays out ``[hi | hi | lo]`` along the columns of A and ``[hi ; lo ; hi]`` along the
+    rows of B, so one bf16 GEMM with ``k' = 3k`` and an fp32 result is ``hi(a) hi(b) + hi(a) lo(b) + lo(a) hi(b)``: error
+    O(2^-16) per product, below TF32's.  The two scratch operands are contiguous, whatever strides the call had.
+    """
+    import torch
+
+    a, b = bound["a"], bound["b"]
+    m, n, k = int(bound["m"]), int(bound["n"]), int(bound["k"])
+    lib = _C.load()
+    a3 = torch.empty((m, 3 * k), dtype=torch.bfloat16, device=a.device)
+    b3 = torch.empty((3 * k, n), dtype=torch.bfloat16, device=a.device)
+    for src, rows, cols, sr, sc, dst, side in ((a, m, k, bound["stride_am"], bound["stride_ak"], a3, 0),
+                                               (b, k, n, bound["stride_bk"], bound["stride_bn"], b3, 1)):
+        status = lib.tnx_split_f32(src.data_ptr(), rows, cols, int(sr), int(sc), dst.data_ptr(), side, stream)
+        if status != _C.OK:
+            raise RuntimeError(f"tnx_split_f32: {_C.strerror(status)}")
+    out = dict(bound)
+    out.update(a=a3, b=b3, k=3 * k, stride_am=3 * k, stride_ak=1, stride_bk=n, stride_bn=1)
+    return out
 
 
 class _BoundLaunch:
@@ -180,6 +225,11 @@ class HipKernel:
             hook(*args, **kwargs)
 
         lib = _C.load()
+        if a.dtype == torch.float32 and b.dtype == torch.float32:
+            if c.dtype != torch.float32:
+                raise ValueError(f"{self.__name__}: float32 operands give a float32 result, got c of {c.dtype}")
+            with torch.cuda.device(a.device):
+                bound = split_f32_operands(bound, torch.cuda.current_stream(a.device).cuda_stream)
         g = self.make_args(bound)
         if a.device.index != torch.cuda.current_device():
             with torch.cuda.device(a.device):
@@ -215,6 +265,9 @@ class HipKernel:
 
         bound = self._bind(args, kwargs)
         lib = _C.load()
+        if bound["a"].dtype == torch.float32:
+            raise ValueError(f"{self.__name__}.prepare binds 16-bit and int8 launches; a float32 call splits its operands "
+                             "on every launch")
         g = self.make_args(bound)
         device = bound["a"].device
         stream = torch.cuda.current_stream(device).cuda_stream

@@ -10,7 +10,7 @@ _conv2d_module = importlib.import_module("tritonix_amd.ops.conv2d")
 __all__ = []
 for _module, _names in ((_matmul_module, ("matmul", "triton_matmul", "hip_matmul", "matmul_splitk", "matmul_kernel",
                                            "gemm_splitk_kernel")),
-                        (_swiglu_module, ("glu_kernel", "glu", "swiglu", "swiglu_ffn", "fused_glu")),
+                        (_swiglu_module, ("glu_kernel", "swiglu_kernel", "glu", "swiglu", "swiglu_ffn", "fused_glu")),
                         (_conv2d_module, ("conv2d_forward", "conv2d_forward_kernel", "torch_conv2d_forward"))):
     for _name in _names:
         globals()[_name] = getattr(_module, _name)

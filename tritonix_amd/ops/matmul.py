@@ -18,9 +18,11 @@ Deliberate differences:
     (row-major, 16-byte aligned rows and base pointers, or anything else) as
     well as (m, n, k): one process runs f16, bf16 and int8 problems, and most
     tiles exist only with the direct-to-LDS loader that needs the first class;
-  * ``matmul`` races HIP variants only (tuned tile, split-K, the 16-row
-    kernel); ``torch.matmul`` is registered un-raced, for ``force_backend``;
-  * int8 inputs give an int32 result;
+  * ``matmul`` keeps the backend names "triton" and "pytorch"; only "triton" (the
+    HIP engine, which settles tile against K split in its own config memo) is
+    timed, ``torch.matmul`` is registered un-raced, for ``force_backend``;
+  * int8 inputs give an int32 result; float32 inputs run as a three-term bf16 split with an fp32 result
+    (``tritonix_amd.kernel.split_f32_operands``) where the reference multiplies them in TF32;
   * split-K sums fp32 partials from a workspace and rounds once, where the
     reference rounds each partial to the output dtype and adds atomically
     (tritonix/ops/matmul.py:195-202); the ``_zero_output`` hook is gone with it.
@@ -249,12 +251,18 @@ def default_config(a, b, split=False):
     g = _C.GemmArgs()
     g.m, g.k = a.shape
     g.n = b.shape[1]
-    g.stride_am, g.stride_ak = a.stride()
-    g.stride_bk, g.stride_bn = b.stride()
-    g.in_dtype = _torch_dtype_code(a.dtype)
-    # base-pointer alignment decides between the two loaders; CPU tensors (host-side planning) count as aligned
-    g.a = a.data_ptr() if a.is_cuda else None
-    g.b = b.data_ptr() if b.is_cuda else None
+    if a.dtype == torch.float32:
+        # what the launch turns a float32 problem into: contiguous bf16 operands, three terms along K, fp32 result
+        g.k = 3 * g.k
+        g.stride_am, g.stride_ak, g.stride_bk, g.stride_bn = g.k, 1, g.n, 1
+        g.in_dtype, g.out_dtype = _C.BF16, _C.F32
+    else:
+        g.stride_am, g.stride_ak = a.stride()
+        g.stride_bk, g.stride_bn = b.stride()
+        g.in_dtype = _torch_dtype_code(a.dtype)
+        # base-pointer alignment decides between the two loaders; CPU tensors (host-side planning) count as aligned
+        g.a = a.data_ptr() if a.is_cuda else None
+        g.b = b.data_ptr() if b.is_cuda else None
     _C.load().tnx_gemm_default_config(ctypes.byref(g))
     cfg = {"block_m": g.block_m, "block_n": g.block_n, "block_k": g.block_k, "group_m": g.group_m,
            "num_stages": g.num_stages, "num_warps": g.num_warps}
@@ -276,17 +284,53 @@ def _autotune_enabled() -> bool:
     return os.environ.get("TRITONIX_AUTOTUNE", "1") not in ("0", "false", "False")
 
 
+def _compute_units(device) -> int:
+    """Workgroups of the large tiles that run together: the CU count of the device."""
+    try:
+        return int(torch.cuda.get_device_properties(device).multi_processor_count)
+    except (RuntimeError, AssertionError):
+        return 256
+
+
+def _tile_or_split(a, b, key):
+    """Config of ``triton_matmul`` for ``key``: the tuned tile, or -- for a problem whose output tiles alone leave
+    CUs idle (fewer 64x128 tiles than the device has CUs) -- whichever of the tuned tile and the tuned K split is
+    faster on these very operands.  Both are configs of the same engine, so the variant a shape ends up on lives
+    in the config memo (and in the tuned-config record on disk), not in the dispatcher: its winner names stay the
+    reference's two, ``"triton"`` and ``"pytorch"`` (tritonix/ops/matmul.py:291-293)."""
+    from tritonix_amd.testing import do_bench
+
+    tile = _tuned_or_tune("matmul", key, matmul_kernel, lambda cfg: _launch_matmul(a, b, cfg), lambda: default_config(a, b))
+    m, n = a.shape[0], b.shape[1]
+    if not _autotune_enabled() or "split_k" in tile or cdiv(m, 64) * cdiv(n, 128) >= _compute_units(a.device):
+        return tile
+    try:
+        cut = _tuned_or_tune("matmul_cut", key, gemm_splitk_kernel, lambda cfg: _launch_splitk(a, b, cfg),
+                             lambda: default_config(a, b, split=True))
+        t_tile = do_bench(lambda: _launch_matmul(a, b, tile), **TUNE_OPTIONS)
+        t_cut = do_bench(lambda: _launch_matmul(a, b, cut), **TUNE_OPTIONS)
+    except (ValueError, RuntimeError):
+        return tile
+    if t_cut < t_tile:
+        save_tuned("matmul", key, cut)
+        return cut
+    return tile
+
+
 def triton_matmul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """C = A @ B on the HIP tile kernel, tile config tuned once per (m, n, k, dtype, layout class).
 
     Keeps the reference's name: callers and the ``"triton"`` backend label of
-    ``matmul`` refer to it.  ``hip_matmul`` is the same function.
+    ``matmul`` refer to it.  ``hip_matmul`` is the same function.  For thin problems the tuned config may carry a
+    K split (``_tile_or_split``).
     """
     _check_2d(a, b)
     a, b = dma_operands(a, b)
     m, k = a.shape
     _, n = b.shape
     key = (m, n, k, a.dtype, dma_layout(a, b))
+    if key not in _matmul_cfg:
+        _matmul_cfg[key] = _tile_or_split(a, b, key)
     return run_memoised(_matmul_cfg, "matmul", key, matmul_kernel, lambda cfg: _launch_matmul(a, b, cfg),
                         lambda: default_config(a, b))
 
@@ -315,24 +359,20 @@ SKINNY_CONFIG = {"block_m": 16, "block_n": 32, "block_k": 32, "group_m": 8, "spl
 
 
 def matmul_skinny(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """C = A @ B for at most 16 rows on the wavefront-level split-K kernel; ``ValueError`` for any other shape."""
+    """C = A @ B for at most 16 rows on the wavefront-level split-K kernel; ``ValueError`` for any other shape.
+
+    Callable on its own; neither ``matmul`` nor ``triton_matmul`` selects it: a workgroup that keeps all of K to
+    itself can own 32 columns at most before the 256 CUs run out of workgroups, and 64-byte row segments stream
+    B at a quarter of what the cross-workgroup hand-over of the tile kernel reaches on the same shape."""
     _check_2d(a, b)
     return _launch_splitk(a, b, SKINNY_CONFIG)
 
 
-def _splitk_backend(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """``matmul_splitk`` as a contender of the dispatcher: only for problems whose output tiles alone leave CUs
-    idle (fewer 64x128 tiles than the part has CUs); any other problem drops out of the race."""
-    _check_2d(a, b)
-    if cdiv(a.shape[0], 64) * cdiv(b.shape[1], 128) >= 256:
-        raise ValueError("the output tiles fill the CUs: no K split is raced for this shape")
-    return matmul_splitk(a, b)
-
-
-# The dispatcher selects among HIP variants only.  ``torch.matmul`` (the reference's "pytorch" backend,
-# tritonix/ops/matmul.py:291-293) is the correctness oracle: ``force_backend("pytorch")`` reaches it, the race
-# never does, so an unforced ``matmul(a, b)`` always runs a kernel of this library.
-matmul = dynamic_dispatch({"triton": triton_matmul, "splitk": _splitk_backend, "skinny": matmul_skinny},
-                          key=["a", "b"])
+# ``matmul`` keeps the reference's two backends and their names (tritonix/ops/matmul.py:291-293): "triton" is the
+# HIP tile engine (its tile / K-split choice is made inside ``triton_matmul``), "pytorch" is ``torch.matmul``.
+# The race times "triton" only: ``torch.matmul`` is the correctness oracle, reached with
+# ``force_backend("pytorch")`` and never chosen, so an unforced ``matmul(a, b)`` always runs a kernel of this
+# library and ``cache`` / ``timings`` hold no other name than the reference's.
+matmul = dynamic_dispatch({"triton": triton_matmul}, key=["a", "b"])
 matmul.register("pytorch", torch.matmul, raced=False)
 matmul.alias("hip", "triton")
