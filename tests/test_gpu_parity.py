@@ -272,7 +272,9 @@ def test_error_mapping_on_launch(device):
     with pytest.raises(ValueError):
         gemm(a[:, :200].t(), a[:200], cfg(128, 128, 64, 4, 3))   # strided A on a DMA-only tile
     with pytest.raises(ValueError):
-        gemm(a.float(), a.float(), GENERIC)
+        gemm(a.double(), a.double(), GENERIC)         # no float64 path (float32 runs as a bf16 split)
+    with pytest.raises(ValueError):
+        gemm(a.float(), a.float(), cfg(256, 256, 64, 4, 2))      # float32: tiles up to 128x128 only
     with pytest.raises(ValueError):
         gemm(a.cpu(), a.cpu(), GENERIC)
 
