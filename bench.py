@@ -20,7 +20,8 @@ Switches for profiling and for the clock / power evidence:
                      without it the line carries per_config only and `value` is null)
   --operands zeros   all-zero operands of the same shapes: the same instruction stream without data-dependent
                      switching power, so the shader clock stays at its maximum (results are then trivially zero)
-  --splitk-reduce atomic   C3 with the K slices added by fp32 atomics instead of the ordered hand-over (for the A/B)
+  --splitk-reduce atomic   C3 with the K slices added by fp32 atomics instead of the ordered hand-over (for the A/B);
+  --splitk-reduce wave     C3 on the 16-row kernel that cuts K across the eight waves of one workgroup (no hand-over)
   --sustain S        after the timed region, keep launching the headline kernel for S seconds while sampling
                      socket power and shader clock with `amd-smi metric -p -c`; reported under "sustain"
 """
@@ -119,8 +120,9 @@ def parse():
     ap.add_argument("--tune", action="store_true", help="run the grid tuner for each workload instead of the built-in tiles")
     ap.add_argument("--only", default=None, help="comma-separated subset of " + ",".join(ALL))
     ap.add_argument("--operands", choices=("random", "zeros"), default="random")
-    ap.add_argument("--splitk-reduce", choices=("ordered", "atomic"), default="ordered",
-                    help="C3 only: how the K slices meet (ordered = stored apart, summed in slice order; atomic = fp32 atomic adds)")
+    ap.add_argument("--splitk-reduce", choices=("ordered", "atomic", "wave"), default="ordered",
+                    help="C3 only: how the K slices meet (ordered = stored apart, summed in slice order; atomic = fp32 atomic "
+                         "adds; wave = the 16-row kernel whose eight waves cut K inside one workgroup and meet in LDS)")
     ap.add_argument("--sustain", type=float, default=0.0, help="seconds of sustained headline launches with power/clock sampling")
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -504,6 +506,8 @@ def extras(torch, dev, oracle, mm, sg, args, operands, wanted):
         cfg = pick_config(mm.gemm_splitk_kernel, lambda c: mm._launch_splitk(a, bs[0], c), a, bs[0], args.tune, split=True)
         if args.splitk_reduce == "atomic":
             cfg = dict(cfg, atomic_reduce=1)
+        elif args.splitk_reduce == "wave":
+            cfg = dict(mm.SKINNY_CONFIG)          # K cut eight ways inside one workgroup, slices meet in LDS
         c = torch.empty((16, 4096), device=dev, dtype=torch.bfloat16)
         l3 = [mm.gemm_splitk_kernel.prepare(a, bs[i], c, 16, 4096, 14336, 14336, 1, 4096, 1, 4096, 1, **cfg)
               for i in range(nrot)]
