@@ -190,6 +190,8 @@ int tnx_tile_coords(int schedule, int id, int tiles_m, int tiles_n, int group_m,
  * in fp32 -- tighter than TF32's 2^-11.  tnx_split_f32 writes the bf16 operand of that product for one float32
  * matrix src[rows, cols] (element strides stride_r, stride_c), contiguous and row-major in dst:
  *   side 0 (the A operand):  dst[rows, 3 * cols] = [ hi | hi | lo ]      side 1 (the B operand):  dst[3 * rows, cols] = [ hi ; lo ; hi ]
+ *   side 2:  dst[rows, 3 * cols] = [ hi | lo | hi ]  (the partner of side 0 when both operands are cut along their
+ *   columns: conv2d's NCHW input, side 0, and KCRS weight, side 2, both along c_in)
  * so that one tnx_gemm with k' = 3k, in_dtype = TNX_BF16 and out_dtype = TNX_F32 (or a GLU epilogue on top) is the
  * float32 product.  Non-finite elements keep their head and get a zero tail.  dst holds 3 * rows * cols bf16 values.
  * Asynchronous on `stream`; allocates nothing. */
@@ -214,7 +216,7 @@ typedef struct tnx_conv2d_args {
   const void* input;   /* [batch, c_in, h_in, w_in]                                 */
   const void* weight;  /* [c_out, c_in, filter_h, filter_w]                         */
   const void* bias;    /* [c_out] of bias_dtype, or NULL                            */
-  void* output;        /* [batch, c_out, h_out, w_out], same type as the input      */
+  void* output;        /* [batch, c_out, h_out, w_out], same type as the input (binary32 with out_f32) */
   int32_t batch, c_in, h_in, w_in;
   int32_t c_out, filter_h, filter_w;
   int32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
@@ -224,6 +226,10 @@ typedef struct tnx_conv2d_args {
   int32_t group_pixels; /* pixel tiles per L2 group (tl.swizzle2d size_g); 0 = 8    */
   int32_t loader;      /* tnx_conv_loader; 0 = the library chooses                   */
   void* stream;        /* hipStream_t; NULL = the null stream                       */
+  int32_t out_f32;     /* non-zero: `output` is binary32, the fp32 sums (+ bias) unrounded -- what makes a float32
+                          convolution a three-term bf16 one: split the input along its channels with
+                          tnx_split_f32(side 0) and the weight with side 2, tripling c_in.  The register-staged
+                          kernels and the GEMM route write it; the direct-to-LDS kernel is then not taken  */
 } tnx_conv2d_args;
 
 /* How the slabs reach LDS.  Two kernels exist: one stages both operands through registers (any stride, padding,

@@ -191,8 +191,10 @@ def test_conv2d_forward_argument_errors():
         conv.conv2d_forward(x.permute(0, 1, 3, 2), w)
     with pytest.raises(AssertionError):
         conv.conv2d_forward(x, torch.zeros(8, 5, 3, 3, dtype=torch.bfloat16))
-    with pytest.raises(NotImplementedError):
-        conv.conv2d_forward(x.float(), w.float())
+    with pytest.raises(ValueError, match="HIP device"):                # host tensors: there is no CPU path, float32 included
+        conv.conv2d_forward(x.float(), w.float(), config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64))
+    with pytest.raises(ValueError, match="HIP device"):
+        conv.conv2d_forward(x, w, config=dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64))
 
 
 def test_torch_conv2d_forward_is_the_library_routine():

@@ -396,3 +396,75 @@ def test_zero_input_and_identity_filter(device):
     wt[torch.arange(16), torch.arange(16), 1, 1] = 1
     out = conv2d_forward(x, wt, None, (1, 1), (1, 1), (1, 1), config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64))
     assert torch.equal(out, x)
+
+
+# ---- float32 tensors: a three-term bf16 convolution over 3 c_in channels with an fp32 result ------------------
+@pytest.mark.parametrize("name,config", [
+    ("all_asymmetric", dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=32)),
+    ("w_out_14", None),
+    ("7x7_stem_ragged_k", dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64)),
+    ("dilated_wide_pad", dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64)),
+], ids=lambda v: str(v).replace(" ", "") if not isinstance(v, dict) else "tile%dx%d" % (v["BLOCK_SIZE_M"], v["BLOCK_SIZE_N"]))
+def test_float32_conv2d(device, name, config, monkeypatch):
+    """The reference convolves float32 tensors in TF32 (tritonix/ops/conv2d/forward.py:100-103, :231-236).  Here: fp32
+    in, fp32 out, error against the float64 convolution far below a bf16 convolution's."""
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    x, wt, b, stride, padding, dilation = _inputs(CASES[name], torch.float32, seed=21)
+    out = conv2d_forward(x.to(device), wt.to(device), None if b is None else b.to(device), stride, padding, dilation, config=config)
+    assert out.dtype == torch.float32
+    b64 = None if b is None else b.double()
+    ref = torch.nn.functional.conv2d(x.double(), wt.double(), b64, stride, padding, dilation)
+    err = ((out.cpu().double() - ref).abs().max() / ref.abs().max()).item()
+    low = torch.nn.functional.conv2d(x.bfloat16().double(), wt.bfloat16().double(), b64, stride, padding, dilation)
+    bf16 = ((low - ref).abs().max() / ref.abs().max()).item()
+    assert err < 2e-4 and err * 30 < bf16, (err, bf16)
+    assert oracle.within_tolerance(out, _oracle(x, wt, b, stride, padding, dilation))[0]
+
+
+def test_float32_conv2d_1x1_on_the_gemm_route(device, monkeypatch):
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    g = torch.Generator("cpu").manual_seed(23)
+    x, wt, b = torch.randn(3, 96, 14, 14, generator=g), torch.randn(80, 96, 1, 1, generator=g) / 96 ** 0.5, torch.randn(80, generator=g)
+    ref = torch.nn.functional.conv2d(x.double(), wt.double(), b.double())
+    for loader in ("gemm", "registers", "auto"):
+        cfg = dict(BLOCK_SIZE_M=0, BLOCK_SIZE_N=0, BLOCK_SIZE_K=0, LOADER=loader)
+        out = conv2d_forward(x.to(device), wt.to(device), b.to(device), config=cfg)
+        assert out.dtype == torch.float32
+        assert ((out.cpu().double() - ref).abs().max() / ref.abs().max()).item() < 2e-4, loader
+    with pytest.raises(ValueError):                                     # the direct-to-LDS kernel writes 16-bit outputs only
+        conv2d_forward(x.to(device), wt.to(device), None, config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, LOADER="dma"))
+
+
+def test_fp32_output_of_a_16_bit_convolution_rounds_to_the_16_bit_output(device):
+    """`out_f32` hands out the fp32 sums (+ bias) before the one rounding: rounded here, they must be the bits the
+    16-bit kernels write (register-staged kernel and GEMM route; through the C ABI)."""
+    import ctypes
+
+    from tritonix_amd import _C
+
+    lib = _C.load()
+    for name, loader in (("all_asymmetric", _C.CONV_LOADER_REGISTERS), ("3x3_same", _C.CONV_LOADER_REGISTERS), ("pointwise", _C.CONV_LOADER_GEMM)):
+        if name == "pointwise":
+            g = torch.Generator("cpu").manual_seed(29)
+            x, wt, b = torch.randn(2, 64, 9, 9, generator=g).bfloat16(), (torch.randn(48, 64, 1, 1, generator=g) / 8).bfloat16(), torch.randn(48, generator=g).bfloat16()
+            stride, padding, dilation = (1, 1), (0, 0), (1, 1)
+        else:
+            x, wt, b, stride, padding, dilation = _inputs(CASES[name], torch.bfloat16, seed=27)
+        n, c, h, w = x.shape
+        k, _, r, s = wt.shape
+        ho, wo = conv.output_size(h, w, r, s, stride, padding, dilation)
+        xd, wd, bd = x.to(device), wt.to(device), None if b is None else b.to(device)
+        outs = {}
+        for f32 in (0, 1):
+            out = torch.empty(n, k, ho, wo, dtype=torch.float32 if f32 else torch.bfloat16, device=device)
+            a = _C.Conv2dArgs()
+            a.input, a.weight, a.output = xd.data_ptr(), wd.data_ptr(), out.data_ptr()
+            a.bias = None if bd is None else bd.data_ptr()
+            a.batch, a.c_in, a.h_in, a.w_in, a.c_out, a.filter_h, a.filter_w = n, c, h, w, k, r, s
+            (a.stride_h, a.stride_w), (a.pad_h, a.pad_w), (a.dil_h, a.dil_w) = stride, padding, dilation
+            a.dtype, a.bias_dtype, a.loader, a.out_f32 = _C.BF16, _C.BF16, loader, f32
+            a.stream = torch.cuda.current_stream().cuda_stream
+            assert lib.tnx_conv2d_forward(ctypes.byref(a)) == _C.OK, (name, f32)
+            torch.cuda.synchronize()
+            outs[f32] = out
+        assert torch.equal(outs[1].bfloat16().view(torch.int16), outs[0].view(torch.int16)), name

@@ -63,7 +63,7 @@ class Conv2dArgs(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("bias_dtype", ctypes.c_int32),
         ("block_pixels", ctypes.c_int32), ("block_cout", ctypes.c_int32), ("block_k", ctypes.c_int32),
         ("group_pixels", ctypes.c_int32), ("loader", ctypes.c_int32),
-        ("stream", ctypes.c_void_p),
+        ("stream", ctypes.c_void_p), ("out_f32", ctypes.c_int32),
     ]
 
 

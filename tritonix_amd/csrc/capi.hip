@@ -504,11 +504,11 @@ __global__ void split_f32_kernel(const float* src, int64_t rows, int64_t cols, i
   const float rest = v - (float)hi;
   const __bf16 lo = (__builtin_isfinite(rest) && __builtin_isfinite(v)) ? (__bf16)rest : (__bf16)0.0f;
   const uint16_t h = __builtin_bit_cast(uint16_t, hi), l = __builtin_bit_cast(uint16_t, lo);
-  if (side == 0) {
+  if (side == 0 || side == 2) {
     uint16_t* row = dst + i * 3 * cols;
     row[j] = h;
-    row[cols + j] = h;
-    row[2 * cols + j] = l;
+    row[cols + j] = side == 0 ? h : l;
+    row[2 * cols + j] = side == 0 ? l : h;
   } else {
     dst[i * cols + j] = h;
     dst[(rows + i) * cols + j] = l;
@@ -518,7 +518,7 @@ __global__ void split_f32_kernel(const float* src, int64_t rows, int64_t cols, i
 
 extern "C" int tnx_split_f32(const float* src, int64_t rows, int64_t cols, int64_t stride_r, int64_t stride_c, void* dst, int side,
                              void* stream) {
-  if (rows < 0 || cols < 0 || (side != 0 && side != 1)) return TNX_E_INVALID;
+  if (rows < 0 || cols < 0 || side < 0 || side > 2) return TNX_E_INVALID;
   if (rows == 0 || cols == 0) return TNX_OK;
   if (!src || !dst) return TNX_E_INVALID;
   const int64_t total = rows * cols;

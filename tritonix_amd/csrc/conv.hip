@@ -153,6 +153,7 @@ static int check_problem(const tnx_conv2d_args* a, int32_t* h_out, int32_t* w_ou
 static bool dma_problem_ok(const tnx_conv2d_args* a, int h_out, int w_out, bool inspect_ptrs) {
   const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
   if (a->stride_w != 1 || gemm_k % 64 != 0) return false;
+  if (a->out_f32) return false;             // the direct-to-LDS kernel's epilogue writes 16-bit outputs only
   if (dma_cols(a, h_out, w_out) >= (1ll << 31) - 4096) return false;
   if (inspect_ptrs && ((uintptr_t)a->weight & 15)) return false;
   // per-lane DMA offsets of the weight slab are 32-bit
@@ -194,7 +195,7 @@ static void fill_gemm(const tnx_conv2d_args* a, const Resolved& r, tnx_gemm_args
   g->stride_am = a->c_in; g->stride_ak = 1;
   g->stride_bk = hw; g->stride_bn = 1;
   g->stride_cm = hw; g->stride_cn = 1;
-  g->in_dtype = a->dtype; g->out_dtype = a->dtype;
+  g->in_dtype = a->dtype; g->out_dtype = a->out_f32 ? TNX_F32 : a->dtype;
   g->block_m = r.bcout; g->block_n = r.bpix; g->block_k = r.bk;
   g->group_m = 8; g->split_k = 1;
   g->num_stages = r.gemm_stages; g->num_warps = r.gemm_warps;
@@ -202,7 +203,7 @@ static void fill_gemm(const tnx_conv2d_args* a, const Resolved& r, tnx_gemm_args
   g->stream = a->stream;
   x->batch = a->batch;
   x->b_batch_bytes = (int64_t)a->c_in * hw * 2;
-  x->c_batch_bytes = (int64_t)a->c_out * hw * 2;
+  x->c_batch_bytes = (int64_t)a->c_out * hw * (a->out_f32 ? 4 : 2);
   x->bias = a->bias;
   x->bias_dtype = a->bias_dtype;
 }
@@ -302,7 +303,8 @@ static void fill_registers(const tnx_conv2d_args* a, const Resolved& r, ConvPara
   p->group = a->group_pixels > 0 ? a->group_pixels : 8;
   p->bias_dtype = a->bias_dtype;
   p->w_vec_ok = gemm_k % 8 == 0 && ((uintptr_t)a->weight & 15) == 0;
-  p->y_vec_ok = p->hw_out % 4 == 0 && ((uintptr_t)a->output & 7) == 0;
+  p->out_f32 = a->out_f32 != 0;
+  p->y_vec_ok = p->hw_out % 4 == 0 && ((uintptr_t)a->output & (p->out_f32 ? 15 : 7)) == 0;
   p->flat = a->filter_h == 1 && a->filter_w == 1 && a->stride_h == 1 && a->stride_w == 1 && a->pad_h == 0 && a->pad_w == 0;
   *grid = (unsigned)(tiles_pix * tiles_cout);
 }
@@ -372,7 +374,7 @@ extern "C" int tnx_conv2d_forward(const tnx_conv2d_args* a) {
   if (st != TNX_OK) return st;
   if (!a->input || !a->weight || !a->output) return TNX_E_INVALID;
   // 16-bit elements are read and written as such
-  if (((uintptr_t)a->input & 1) || ((uintptr_t)a->weight & 1) || ((uintptr_t)a->output & 1)) return TNX_E_INVALID;
+  if (((uintptr_t)a->input & 1) || ((uintptr_t)a->weight & 1) || ((uintptr_t)a->output & (a->out_f32 ? 3 : 1))) return TNX_E_INVALID;
   if (a->bias && ((uintptr_t)a->bias & (a->bias_dtype == TNX_F32 ? 3 : 1))) return TNX_E_INVALID;
   unsigned grid = 0;
   hipError_t err;

@@ -38,6 +38,7 @@ struct ConvParams {
   bool w_vec_ok;          // weight rows take 16-byte loads: gemm_k % 8 == 0 and a 16-byte aligned base
   bool y_vec_ok;          // four consecutive pixels lie in one plane and take one 8-byte store: hw_out % 4 == 0, aligned base
   bool flat;              // 1x1 filter, unit strides, no padding: all pixels of one image plane are contiguous in the input
+  bool out_f32;           // y is binary32: the fp32 sums (+ bias) as they are (y_vec_ok then means one 16-byte store)
 };
 
 typedef hipError_t (*conv_launch_fn)(const ConvParams& p, unsigned grid, hipStream_t stream);
@@ -328,6 +329,24 @@ __global__ __launch_bounds__(C::THREADS, TNX_CONV_OCC) void conv2d_tile_kernel(C
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + wx * C::WTN + j * MI + (lane / MI) * 4;
       if (n >= p.pixels) continue;
+      if (p.out_f32) {
+        float* y32 = (float*)p.y;
+        if (p.y_vec_ok) {
+          const int img = (int)fd_div((uint32_t)n, p.div_hw_out);
+          const int r0 = n - img * p.hw_out;
+          const f32x4 v = {acc[i][j][0] + bv, acc[i][j][1] + bv, acc[i][j][2] + bv, acc[i][j][3] + bv};
+          __builtin_nontemporal_store(v, (f32x4*)(y32 + ((int64_t)img * p.c_out + row) * p.hw_out + r0));
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (n + r >= p.pixels) break;
+            const int img = (int)fd_div((uint32_t)(n + r), p.div_hw_out);
+            const int r0 = n + r - img * p.hw_out;
+            y32[((int64_t)img * p.c_out + row) * p.hw_out + r0] = acc[i][j][r] + bv;
+          }
+        }
+        continue;
+      }
       typename O::raw out[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) out[r] = O::cvt(acc[i][j][r] + bv);

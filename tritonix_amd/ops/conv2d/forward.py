@@ -5,8 +5,9 @@
 str_w, pad_h, pad_w, dil_h, dil_w, GEMM_M, GEMM_N, GEMM_K, BLOCK_SIZE_M=, BLOCK_SIZE_N=, BLOCK_SIZE_K=,
 GROUP_SIZE_M=, OUT_DTYPE=, USE_TF32=)`` keep the argument order and meaning of
 tritonix/ops/conv2d/forward.py:19-48 and :202-311; both end in one ``tnx_conv2d_forward`` through the C ABI on
-torch's current stream.  Float16 and bfloat16 are built; float32 input (the reference's TF32 mode) raises, since
-gfx950 has no TF32 matrix instruction.
+torch's current stream.  Float16 and bfloat16 are built; float32 tensors (the reference convolves them in TF32,
+which gfx950 has no matrix instruction for) run as a three-term bf16 convolution over 3 c_in channels with an fp32
+result (``_split_f32``), on the register-staged kernels and the 1x1 GEMM route.
 """
 from __future__ import annotations
 
@@ -51,6 +52,23 @@ def output_size(h_in: int, w_in: int, filter_h: int, filter_w: int, stride, padd
     return h_out, w_out
 
 
+def _split_f32(x, w, batch, c_in, h_in, w_in, c_out, filter_h, filter_w):
+    """float32 input and weight as the bf16 tensors of a three-term product (the reference convolves float32 in
+    TF32, tritonix/ops/conv2d/forward.py:100-103; gfx950 has no TF32 matrix instruction): both are cut into a bf16 head
+    and tail along the input channels, ``x -> [hi | hi | lo]`` (3 c_in channels) and ``w -> [hi | lo | hi]``, so that the
+    ordinary bf16 convolution over 3 c_in channels with an fp32 result is ``hi hi + hi lo + lo hi``.  Returns
+    ``(x3, w3, 3 * c_in)``."""
+    lib = _C.load()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    x3 = torch.empty((batch, 3 * c_in, h_in, w_in), dtype=torch.bfloat16, device=x.device)
+    w3 = torch.empty((c_out, 3 * c_in, filter_h, filter_w), dtype=torch.bfloat16, device=x.device)
+    for src, rows, cols, dst, side in ((x, batch, c_in * h_in * w_in, x3, 0), (w, c_out, c_in * filter_h * filter_w, w3, 2)):
+        status = lib.tnx_split_f32(src.data_ptr(), rows, cols, cols, 1, dst.data_ptr(), side, stream)
+        if status != _C.OK:
+            raise RuntimeError(f"tnx_split_f32: {_C.strerror(status)}")
+    return x3, w3, 3 * c_in
+
+
 def _raise_for_status(status: int, a: _C.Conv2dArgs) -> None:
     if status == _C.OK:
         return
@@ -71,6 +89,12 @@ def _raise_for_status(status: int, a: _C.Conv2dArgs) -> None:
 def _args(out, input, weight, bias, batch, c_in, h_in, w_in, c_out, filter_h, filter_w, stride, padding, dilation,
           block_m: int, block_n: int, block_k: int, group_m: int, loader: int = 0) -> _C.Conv2dArgs:
     a = _C.Conv2dArgs()
+    if not (input.is_cuda and weight.is_cuda and out.is_cuda):
+        raise ValueError("conv2d_forward: input, weight and output must be tensors on a HIP device (there is no CPU path)")
+    if input.dtype == torch.float32:
+        input, weight, c_in = _split_f32(input, weight, batch, c_in, h_in, w_in, c_out, filter_h, filter_w)
+        a.out_f32 = 1
+        a._keep = (input, weight)              # the scratch operands live as long as the bound arguments
     a.input, a.weight, a.output = input.data_ptr(), weight.data_ptr(), out.data_ptr()
     a.bias = bias.data_ptr() if bias is not None else None
     a.batch, a.c_in, a.h_in, a.w_in = batch, c_in, h_in, w_in
@@ -79,7 +103,7 @@ def _args(out, input, weight, bias, batch, c_in, h_in, w_in, c_out, filter_h, fi
     a.pad_h, a.pad_w = padding
     a.dil_h, a.dil_w = dilation
     if input.dtype not in _DTYPES:
-        raise ValueError(f"conv2d_forward: dtype {input.dtype} has no HIP kernel (float16 and bfloat16 are built)")
+        raise ValueError(f"conv2d_forward: dtype {input.dtype} has no HIP kernel (float16, bfloat16 and float32 are built)")
     a.dtype = _DTYPES[input.dtype]
     if bias is not None:
         if bias.dtype not in _DTYPES:
@@ -157,6 +181,8 @@ class Conv2dForwardKernel:
         """Bind once, launch many times: a callable that re-issues the same ``tnx_conv2d_forward`` (on the stream that
         was current when ``prepare`` ran)."""
         a = self.bind(*args, **kwargs)
+        if a.out_f32:
+            raise ValueError("conv2d_forward_kernel.prepare binds 16-bit launches; a float32 call splits its operands on every launch")
         fn = _C.load().tnx_conv2d_forward
         ref = ctypes.byref(a)
 
@@ -233,9 +259,6 @@ def conv2d_forward(
     stride, padding, dilation = tuple(stride), tuple(padding), tuple(dilation)
     h_out, w_out = output_size(h_in, w_in, r, s, stride, padding, dilation)
     gemm_m, gemm_n, gemm_k = n * h_out * w_out, c_out, c_in * r * s
-    if input.dtype == torch.float32:
-        raise NotImplementedError("conv2d_forward is built for float16 and bfloat16; float32 (TF32) input has no "
-                                  "matrix instruction on gfx950")
     out = input.new_empty((n, c_out, h_out, w_out))
 
     def launch(bm, bn, bk, g, loader="auto", dst=out):
