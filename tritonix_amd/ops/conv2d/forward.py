@@ -89,9 +89,9 @@ def _raise_for_status(status: int, a: _C.Conv2dArgs) -> None:
 def _args(out, input, weight, bias, batch, c_in, h_in, w_in, c_out, filter_h, filter_w, stride, padding, dilation,
           block_m: int, block_n: int, block_k: int, group_m: int, loader: int = 0) -> _C.Conv2dArgs:
     a = _C.Conv2dArgs()
-    if not (input.is_cuda and weight.is_cuda and out.is_cuda):
-        raise ValueError("conv2d_forward: input, weight and output must be tensors on a HIP device (there is no CPU path)")
     if input.dtype == torch.float32:
+        if not (input.is_cuda and weight.is_cuda and out.is_cuda):
+            raise ValueError("conv2d_forward: input, weight and output must be tensors on a HIP device (there is no CPU path)")
         input, weight, c_in = _split_f32(input, weight, batch, c_in, h_in, w_in, c_out, filter_h, filter_w)
         a.out_f32 = 1
         a._keep = (input, weight)              # the scratch operands live as long as the bound arguments
@@ -174,6 +174,9 @@ class Conv2dForwardKernel:
                      b["GROUP_SIZE_M"], _LOADERS[b.get("LOADER", "auto")])
 
     def run(self, *args, grid=None, **kwargs):
+        for t in args[:3]:
+            if isinstance(t, torch.Tensor) and not t.is_cuda:
+                raise ValueError("conv2d_forward_kernel: output, input and weight must be tensors on a HIP device (there is no CPU path)")
         a = self.bind(*args, **kwargs)
         _raise_for_status(_C.load().tnx_conv2d_forward(ctypes.byref(a)), a)
 
