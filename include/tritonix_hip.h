@@ -228,8 +228,7 @@ typedef struct tnx_conv2d_args {
   void* stream;        /* hipStream_t; NULL = the null stream                       */
   int32_t out_f32;     /* non-zero: `output` is binary32, the fp32 sums (+ bias) unrounded -- what makes a float32
                           convolution a three-term bf16 one: split the input along its channels with
-                          tnx_split_f32(side 0) and the weight with side 2, tripling c_in.  The register-staged
-                          kernels and the GEMM route write it; the direct-to-LDS kernel is then not taken  */
+                          tnx_split_f32(side 0) and the weight with side 2, tripling c_in                    */
 } tnx_conv2d_args;
 
 /* How the slabs reach LDS.  Two kernels exist: one stages both operands through registers (any stride, padding,

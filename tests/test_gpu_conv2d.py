@@ -431,8 +431,20 @@ def test_float32_conv2d_1x1_on_the_gemm_route(device, monkeypatch):
         out = conv2d_forward(x.to(device), wt.to(device), b.to(device), config=cfg)
         assert out.dtype == torch.float32
         assert ((out.cpu().double() - ref).abs().max() / ref.abs().max()).item() < 2e-4, loader
-    with pytest.raises(ValueError):                                     # the direct-to-LDS kernel writes 16-bit outputs only
-        conv2d_forward(x.to(device), wt.to(device), None, config=dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, LOADER="dma"))
+
+
+def test_float32_conv2d_on_the_direct_to_lds_kernel(device):
+    """3 * 64 * 9 = 27 K slabs of 64: the split problem fits the DMA ring; same sums in the same order as the
+    register-staged kernel, so the two float32 outputs agree bit for bit."""
+    g = torch.Generator("cpu").manual_seed(31)
+    x, wt, b = torch.randn(2, 64, 14, 14, generator=g), torch.randn(128, 64, 3, 3, generator=g) / 24, torch.randn(128, generator=g)
+    xd, wd, bd = x.to(device), wt.to(device), b.to(device)
+    tile = dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64)
+    dma = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1), config=dict(tile, LOADER="dma"))
+    reg = conv2d_forward(xd, wd, bd, (1, 1), (1, 1), (1, 1), config=dict(tile, LOADER="registers"))
+    assert dma.dtype == torch.float32 and torch.equal(dma, reg)
+    ref = torch.nn.functional.conv2d(x.double(), wt.double(), b.double(), (1, 1), (1, 1))
+    assert ((dma.cpu().double() - ref).abs().max() / ref.abs().max()).item() < 2e-4
 
 
 def test_fp32_output_of_a_16_bit_convolution_rounds_to_the_16_bit_output(device):

@@ -153,7 +153,6 @@ static int check_problem(const tnx_conv2d_args* a, int32_t* h_out, int32_t* w_ou
 static bool dma_problem_ok(const tnx_conv2d_args* a, int h_out, int w_out, bool inspect_ptrs) {
   const int64_t gemm_k = (int64_t)a->c_in * a->filter_h * a->filter_w;
   if (a->stride_w != 1 || gemm_k % 64 != 0) return false;
-  if (a->out_f32) return false;             // the direct-to-LDS kernel's epilogue writes 16-bit outputs only
   if (dma_cols(a, h_out, w_out) >= (1ll << 31) - 4096) return false;
   if (inspect_ptrs && ((uintptr_t)a->weight & 15)) return false;
   // per-lane DMA offsets of the weight slab are 32-bit
@@ -326,7 +325,7 @@ static void fill_dma(const tnx_conv2d_args* a, const Resolved& r, GemmParams* p,
   p->group_m = 8;            // with one or two channel tiles: the channel tiles of one pixel tile run side by side
   p->split_k = 1;
   p->ktiles_per_split = (int)(gemm_k / r.bk);
-  p->out_dtype = a->dtype;
+  p->out_dtype = a->out_f32 ? TNX_F32 : a->dtype;
   ConvGeom& g = p->cv;
   g.h_in = im.h_in; g.w_in = im.w_in; g.c_out = a->c_out; g.h_out = h_out; g.w_out = w_out; g.wp = wp;
   g.stride_h = a->stride_h; g.pad_h = a->pad_h; g.pad_w = a->pad_w;

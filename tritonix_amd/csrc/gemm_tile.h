@@ -853,17 +853,16 @@ struct __attribute__((packed, aligned(2))) Loose16 {
 template <class T, class C, class O, class ACC>
 __device__ __forceinline__ void epilogue_store_conv(ACC (&acc)[C::TM][C::TN], uint8_t* ybase, uint32_t lds_strip, int lane,
                                                     int gm0, int gn0, const ConvGeom& g) {
-  typedef Pack16<O, float, false> PK;
-  typedef typename PK::raw raw;
+  typedef typename O::raw raw;                          // 16-bit outputs, or binary32 (the fp32 sums + bias as they are)
   typedef float acc4 __attribute__((ext_vector_type(4)));
   constexpr int MI = C::MI;
   constexpr int NGRP = C::ACC_N / 4;
   constexpr int PITCH = EpiStage<C>::PITCH;
   constexpr int ROWS = EpiStage<C>::ROWS;
-  constexpr int CPRW = C::WTN / PK::OUTV;
+  constexpr int CPRW = C::WTN / 8;                       // a lane handles 8 pixels: one 16-byte chunk of the im2col slab
   constexpr int ITERS = (ROWS * CPRW + 63) / 64;
   constexpr int UNR = ITERS % 4 == 0 ? 4 : (ITERS % 2 == 0 ? 2 : 1);
-  static_assert(EpiStage<C>::RB == 1 && PK::OUTV == 8, "one row-block per pass, 8 outputs per chunk");
+  static_assert(EpiStage<C>::RB == 1 && C::WTN % 8 == 0, "one row-block per pass, 8 outputs per chunk");
   raw* yp = (raw*)ybase;
   const uint32_t wbase = lds_strip + (lane % MI) * PITCH + (lane / MI) * 16;
 #pragma unroll
@@ -910,9 +909,11 @@ __device__ __forceinline__ void epilogue_store_conv(ACC (&acc)[C::TM][C::TN], ui
         for (int x = 0; x < 8; ++x) out[x] = O::cvt(f[u][x] + bv);
         raw* dst = yp + (((int64_t)img * g.c_out + gm) * g.h_out + ho) * g.w_out + wq;
         if (valid >= 8) {
-          i32x4 v;
-          __builtin_memcpy(&v, out, 16);
-          store16_stream_loose(dst, v);    // 2-byte aligned: w_out need not be a multiple of 8
+          i32x4 v[sizeof(raw) / 2];
+          __builtin_memcpy(v, out, 8 * sizeof(raw));
+#pragma unroll
+          for (int h = 0; h < (int)sizeof(raw) / 2; ++h)
+            store16_stream_loose((uint8_t*)dst + 16 * h, v[h]);    // element-aligned: w_out need not be a multiple of 8
         } else {
 #pragma unroll 1
           for (int x = 0; x < valid; ++x) dst[x] = out[x];
@@ -1768,7 +1769,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
     const int64_t gn0 = n0 + wx * C::WTN;
     const uint32_t strip = lds0 + wave * EpiStage<C>::WAVE_BYTES;
     if constexpr (CONV) {
-      epilogue_store_conv<T, C, O>(acc, p.c, strip, lane, (int)gm0, (int)gn0, p.cv);
+      if (p.out_dtype == DT_F32) epilogue_store_conv<T, C, OutF32>(acc, p.c, strip, lane, (int)gm0, (int)gn0, p.cv);
+      else epilogue_store_conv<T, C, O>(acc, p.c, strip, lane, (int)gm0, (int)gn0, p.cv);
       return;
     }
     // the output type: the input's own 16-bit type (int32 for int8), or binary32 where that epilogue is built
