@@ -158,6 +158,29 @@ def test_default_config_is_always_launchable():
                 assert g.tail_tiles == 0 and lib.tnx_gemm_workspace_bytes(ctypes.byref(g)) == 0
 
 
+def test_default_config_on_random_problems_is_launchable_for_every_output_type():
+    """600 problems from a fixed seed, all three input types and, for the 16-bit floats, both output types (the input's
+    own and binary32, the output of a split float32 product): the built-in choice always names a built kernel that
+    takes these operands, within the LDS budget, and a float32 result never lands on a tile without that epilogue."""
+    import random
+
+    lib = _C.load()
+    rng = random.Random(20251)
+    for _ in range(600):
+        m = rng.choice([1, 7, 16, 33, 64, 100, 128, 257, 512, 1000, 2048, 4096, 8192, 12288])
+        n = rng.choice([8, 24, 64, 136, 256, 520, 1024, 3072, 4096, 14336, 28672])
+        k = rng.choice([8, 64, 72, 200, 512, 1032, 4096, 8192, 14336])
+        dt, out = rng.choice([(_C.BF16, _C.BF16), (_C.F16, _C.F16), (_C.I8, _C.I32), (_C.BF16, _C.F32), (_C.F16, _C.F32)])
+        if dt == _C.I8:
+            n, k = -(-n // 16) * 16, -(-k // 16) * 16          # int8 rows of A and B as the DMA loader takes them
+        g = args(m=m, n=n, k=k, stride_am=k, stride_bk=n, stride_cm=n, in_dtype=dt, out_dtype=out)
+        assert lib.tnx_gemm_default_config(ctypes.byref(g)) == _C.OK
+        assert lib.tnx_gemm_supported(ctypes.byref(g)) == _C.OK, (dt, out, m, n, k, g.block_m, g.block_n, g.block_k, g.num_warps, g.num_stages)
+        assert 0 < lib.tnx_gemm_lds_bytes(ctypes.byref(g)) <= _C.LDS_LIMIT_BYTES
+        if out == _C.F32:
+            assert g.block_m * g.block_n <= 128 * 128
+
+
 def test_default_config_of_the_benchmark_shapes():
     lib = _C.load()
 

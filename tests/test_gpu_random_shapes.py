@@ -84,3 +84,50 @@ def test_random_problems_on_random_tiles(device, seed):
         bound = 1e-2 * ref.abs() + 1e-2 * ref.pow(2).mean().sqrt() + 1e-3
         assert bool(((got - ref).abs() <= bound).all()), what
     assert ran == 120
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_float32_problems(device, seed):
+    """float32 operands (a three-term bf16 split inside the launch) on every tile that carries the fp32 epilogue:
+    NaN-embedded strided views, both layouts, K cuts and the gated epilogue; error bound 2e-4 of the largest result
+    against the float64 product, fifty times tighter than the 16-bit bar."""
+    rnd = random.Random(100 + seed)
+    tiles = []
+    for name in _C.kernel_names():
+        f = name.split()
+        if f[0] == "bf16" and int(f[1]) * int(f[2]) <= 128 * 128:
+            tiles.append(tuple(int(v) for v in f[1:6]) + ("bt" in f[6:],))
+    assert tiles
+    for case in range(60):
+        bm, bn, bk, nw, st, _ = rnd.choice(tiles)
+        m = rnd.choice([1, 5, 16, 64, 100, 257, 513])
+        n = rnd.choice([8, 24, 100, 256, 264, 1000])
+        k = rnd.choice([1, 7, 40, 64, 200, 517, 1024])
+        layout = rnd.choice(["row-major", "row-major", "k-contiguous", "column-major-a"])
+        glu = rnd.random() < 0.2 and n % 2 == 0
+        split = 1 if glu else rnd.choice([1, 1, 2, 4])
+        g = torch.Generator("cpu").manual_seed(5000 * seed + case)
+        a = torch.randn(m, k, generator=g)
+        b = torch.randn(k, n, generator=g) / k ** 0.5
+        fill = float("nan")
+        ad = embedded(a, rnd.choice([0, 1, 3]), rnd.choice([0, 1, 8]), fill, device) if layout != "column-major-a" else \
+            embedded(a.t().contiguous(), 1, 2, fill, device).t()
+        bd = embedded(b, rnd.choice([0, 5]), rnd.choice([0, 3]), fill, device) if layout != "k-contiguous" else \
+            embedded(b.t().contiguous(), 2, 1, fill, device).t()
+        cfg = dict(block_m=bm, block_n=bn, block_k=bk, group_m=8, num_stages=st, num_warps=nw)
+        if split > 1:
+            cfg["split_k"] = split
+        what = f"seed {seed} case {case}: f32 {m}x{n}x{k} {layout}, {cfg}, glu {glu}"
+        if glu:
+            out = sg._launch_glu(ad, bd, cfg, "silu")
+        elif split > 1:
+            out = mm._launch_splitk(ad, bd, cfg)
+        else:
+            out = mm._launch_matmul(ad, bd, cfg)
+        torch.cuda.synchronize()
+        assert out.dtype == torch.float32, what
+        y = a.double() @ b.double()
+        ref = torch.nn.functional.silu(y[:, 0::2]) * y[:, 1::2] if glu else y
+        got = out.cpu().double()
+        assert bool(torch.isfinite(got).all()), what
+        assert float((got - ref).abs().max()) <= 2e-4 * max(float(ref.abs().max()), 1e-3) * (3 if glu else 1), what
