@@ -30,6 +30,14 @@
 #ifndef TNX_LADDER
 #define TNX_LADDER 0
 #endif
+// Development schedule (never the shipped library): -D TNX_PINGPONG=1 runs the K loop of the eight-wave two-slot
+// tiles with two k steps per slab as a ping-pong: the two waves of every SIMD alternate, a barrier apart, between
+// reading a whole slab's fragments from LDS and multiplying them at raised priority (see pingpong_loop).  Values
+// above 1 are its attribution forms: 2 priority not raised; 3 without the fragment reads, 4 without the DMA refill,
+// 5 without the MFMAs (3-5: wrong results on purpose).  Measured, it loses to the interleaved loop on every operand.
+#ifndef TNX_PINGPONG
+#define TNX_PINGPONG 0
+#endif
 
 namespace tnx {
 
@@ -1035,6 +1043,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   // current one has run, so the epilogue keeps its own copy of the origin.)
   int64_t m0 = 0, n0 = 0;
   uint32_t a_voff[C::A_LPW], b_voff[C::B_LPW];
+  constexpr bool PINGPONG_TILE = TNX_PINGPONG && FAST && !PERSIST && !BT && !CONV && NW == 8 && STAGES == 2 && C::KSTEPS == 2;
   // CONV: a lane's B ops all fetch the same 16-byte LDS column slot; the pixel chunk that lands there is one of
   // two (the LDS swizzle moves it by two chunks depending on the k row): element offset of (image, channel 0,
   // h0, w0) and the packed (h0, w0) for both, (h0, w0) being the input position of filter tap (0, 0).  Pixels past
@@ -1738,13 +1747,103 @@ __global__ __launch_bounds__(C::THREADS) void gemm_tile_kernel(GemmParams p) {
   }
   };
 
+  // Ping-pong form of the K loop (TNX_PINGPONG builds).  The waves 0..NW/2-1 ("lead") and NW/2..NW-1 share the SIMDs
+  // pairwise.  Time runs in phases 0..2*KT, a workgroup barrier before each; slab v takes two of them:
+  //   phase 2v     lead: reads both k steps' fragments of slab v from LDS      other: the MFMAs of slab v-1
+  //                both: issue their DMA ops of slab v+1 into the slot slab v-1 has left (read last in phase 2v-1)
+  //   phase 2v+1   lead: the MFMAs of slab v, priority raised                   other: reads slab v; all wait for the DMA
+  // and phase 2*KT for the second group's last slab.  Each group runs its own straight loop; both execute 2*KT+1
+  // barriers.  Needs an even KT >= 2 (the prologue has issued slabs 0 and 1); the caller falls back to k_loop().
+  auto pingpong_loop = [&]() __attribute__((always_inline)) {
+    constexpr int NRD = C::KSTEPS * NREAD, NMM = C::KSTEPS * NMMA;
+    auto load_phase = [&](uint32_t sa, auto with_dma, uint32_t dst) __attribute__((always_inline)) {
+      constexpr bool WITH_DMA = decltype(with_dma)::value;
+      // opaque slot base: the lane addresses of the phase are formed here and die with it, instead of one set per
+      // slot living in registers through every phase
+      asm volatile("" : "+s"(sa));
+      const uint32_t sb = sa + C::A_BYTES;
+#pragma unroll
+      for (int i = 0; i < NRD; ++i) {
+        if (TNX_PINGPONG != 3) read_one(i / NREAD, i % NREAD, sa, sb, i / NREAD);
+        if constexpr (WITH_DMA) {
+#pragma unroll
+          for (int q = i * C::LPW / NRD; q < (i + 1) * C::LPW / NRD; ++q) if (TNX_PINGPONG != 4) dma_op(q, dst);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (WITH_DMA) dma_advance();
+      __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the slot may be refilled after the next barrier
+    };
+    auto mma_phase = [&](auto with_dma, uint32_t dst) __attribute__((always_inline)) {
+      constexpr bool WITH_DMA = decltype(with_dma)::value;
+      constexpr int HALF = NMM / 2;         // the refill goes out under the first half of the MFMAs
+      if (TNX_PINGPONG != 2) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int i = 0; i < NMM; ++i) {
+        if (TNX_PINGPONG != 5) mma_one(i / NMMA, i % NMMA);
+        if constexpr (WITH_DMA) {
+          if (i < HALF) {
+#pragma unroll
+            for (int q = i * C::LPW / HALF; q < (i + 1) * C::LPW / HALF; ++q) if (TNX_PINGPONG != 4) dma_op(q, dst);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_setprio(0);
+      if constexpr (WITH_DMA) dma_advance();
+    };
+    auto phase_barrier = [&]() __attribute__((always_inline)) {
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    const uint32_t s0 = lds0, s1 = lds0 + C::STAGE_BYTES;
+    if (wave < NW / 2) {
+      for (int v = 0; v < KT; v += 2) {
+        phase_barrier();                                             // phase 2v
+        if (v > 0) load_phase(s0, Yes{}, s1); else load_phase(s0, No{}, 0u);
+        phase_barrier();                                             // 2v+1
+        mma_phase(No{}, 0u);
+        TNX_WAIT_VM(0);
+        phase_barrier();                                             // 2v+2
+        if (v + 2 < KT) load_phase(s1, Yes{}, s0); else load_phase(s1, No{}, 0u);
+        phase_barrier();                                             // 2v+3
+        mma_phase(No{}, 0u);
+        TNX_WAIT_VM(0);
+      }
+      phase_barrier();                                               // phase 2*KT: the other group's last MFMAs
+    } else {
+      phase_barrier();                                               // phase 0: nothing to multiply yet
+      for (int v = 0; v + 2 < KT; v += 2) {
+        phase_barrier();                                             // 2v+1
+        load_phase(s0, No{}, 0u);
+        TNX_WAIT_VM(0);
+        phase_barrier();                                             // 2v+2: slab v, and the DMA of slab v+2
+        mma_phase(Yes{}, s0);
+        phase_barrier();                                             // 2v+3
+        load_phase(s1, No{}, 0u);
+        TNX_WAIT_VM(0);
+        phase_barrier();                                             // 2v+4: slab v+1, and the DMA of slab v+3
+        mma_phase(Yes{}, s1);
+      }
+      phase_barrier();                                               // the last two slabs: nothing left to fetch
+      load_phase(s0, No{}, 0u);
+      TNX_WAIT_VM(0);
+      phase_barrier();
+      mma_phase(No{}, 0u);
+      phase_barrier();
+      load_phase(s1, No{}, 0u);
+      phase_barrier();                                               // phase 2*KT
+      mma_phase(No{}, 0u);
+    }
+  };
   typedef typename OutOf<T>::type O;
   if constexpr (!PERSIST) {
     if (KT > 0) {
       issue_prologue();
       if (KT >= STAGES) { TNX_WAIT_VM((STAGES - 1) * C::LPW); } else { TNX_WAIT_VM(0); }
     }
-    k_loop();
+    if (PINGPONG_TILE && KT >= 2 && (KT & 1) == 0) pingpong_loop();
+    else k_loop();
     if constexpr (FAST && !CONV) {
       if (tail_here) {
         // the left-out slab: every wave is done with the ring, slot 0 takes it, one slab of MFMAs follows
