@@ -193,7 +193,9 @@ int tnx_tile_coords(int schedule, int id, int tiles_m, int tiles_n, int group_m,
  *   side 2:  dst[rows, 3 * cols] = [ hi | lo | hi ]  (the partner of side 0 when both operands are cut along their
  *   columns: conv2d's NCHW input, side 0, and KCRS weight, side 2, both along c_in)
  * so that one tnx_gemm with k' = 3k, in_dtype = TNX_BF16 and out_dtype = TNX_F32 (or a GLU epilogue on top) is the
- * float32 product.  Non-finite elements keep their head and get a zero tail.  dst holds 3 * rows * cols bf16 values.
+ * float32 product.  A non-finite element is carried by the first copy of its head alone: its tail and the second copy
+ * of its head (the one multiplied with the other operand's tail) are zero, so inf * finite stays inf and does not
+ * become inf + inf * 0 = NaN.  dst holds 3 * rows * cols bf16 values.
  * Asynchronous on `stream`; allocates nothing. */
 int tnx_split_f32(const float* src, int64_t rows, int64_t cols, int64_t stride_r, int64_t stride_c, void* dst, int side,
                   void* stream);

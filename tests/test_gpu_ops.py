@@ -279,19 +279,44 @@ def test_split_f32_lays_out_head_and_tail(device):
     x = torch.randn(37, 53, generator=g) * torch.logspace(-6, 6, 53)
     x[3, 4], x[5, 6], x[7, 8] = float("inf"), float("-inf"), 0.0
     hi, lo = _split_reference(x)
-    lo[3, 4] = lo[5, 6] = 0                                            # non-finite elements keep their head only
+    lo[3, 4] = lo[5, 6] = 0                                            # non-finite elements keep their head only,
+    hi2 = hi.clone()
+    hi2[3, 4] = hi2[5, 6] = 0                                          # and only in its first copy
     xd = x.to(device)
     lib, stream = _C.load(), torch.cuda.current_stream().cuda_stream
     a3 = torch.empty(37, 3 * 53, dtype=torch.bfloat16, device=device)
     b3 = torch.empty(3 * 37, 53, dtype=torch.bfloat16, device=device)
     assert lib.tnx_split_f32(xd.data_ptr(), 37, 53, 53, 1, a3.data_ptr(), 0, stream) == _C.OK
     assert lib.tnx_split_f32(xd.data_ptr(), 37, 53, 53, 1, b3.data_ptr(), 1, stream) == _C.OK
-    assert torch.equal(a3.cpu().view(torch.int16), torch.cat([hi, hi, lo], dim=1).view(torch.int16))
-    assert torch.equal(b3.cpu().view(torch.int16), torch.cat([hi, lo, hi], dim=0).view(torch.int16))
+    assert torch.equal(a3.cpu().view(torch.int16), torch.cat([hi, hi2, lo], dim=1).view(torch.int16))
+    assert torch.equal(b3.cpu().view(torch.int16), torch.cat([hi, lo, hi2], dim=0).view(torch.int16))
+    w3 = torch.empty(37, 3 * 53, dtype=torch.bfloat16, device=device)
+    assert lib.tnx_split_f32(xd.data_ptr(), 37, 53, 53, 1, w3.data_ptr(), 2, stream) == _C.OK
+    assert torch.equal(w3.cpu().view(torch.int16), torch.cat([hi, lo, hi2], dim=1).view(torch.int16))
     # a transposed view: strides (1, 53) of the same storage
     t3 = torch.empty(53, 3 * 37, dtype=torch.bfloat16, device=device)
     assert lib.tnx_split_f32(xd.data_ptr(), 53, 37, 1, 53, t3.data_ptr(), 0, stream) == _C.OK
-    assert torch.equal(t3.cpu().view(torch.int16), torch.cat([hi.t(), hi.t(), lo.t()], dim=1).contiguous().view(torch.int16))
+    assert torch.equal(t3.cpu().view(torch.int16), torch.cat([hi.t(), hi2.t(), lo.t()], dim=1).contiguous().view(torch.int16))
+
+
+def test_float32_matmul_keeps_infinities_and_nans_where_fp32_has_them(device, monkeypatch):
+    """inf * finite is inf and inf * 0 is NaN in the fp32 product; the three-term split must not add an inf * 0 of its
+    own (the tail of a value bf16 holds exactly is 0).  Same pattern of inf / -inf / NaN as the CPU fp32 matmul, and
+    the finite entries within the float32 tolerance."""
+    monkeypatch.setenv("TRITONIX_AUTOTUNE", "0")
+    g = torch.Generator("cpu").manual_seed(77)
+    a, b = torch.randn(128, 256, generator=g), torch.randn(256, 192, generator=g) / 16
+    b[:, :8] = b[:, :8].bfloat16().float()                            # columns whose tails are exactly zero
+    b[5, 3] = 1.0
+    a[2, 5], a[9, 100], a[40, 7] = float("inf"), float("-inf"), float("nan")
+    b[17, 150], b[200, 20] = float("inf"), 0.0
+    a[70, 200] = float("inf")                                          # meets b[200, 20] == 0: NaN in fp32 too
+    ref = a @ b
+    out = tritonix_amd.triton_matmul(a.to(device), b.to(device)).cpu()
+    assert torch.equal(torch.isnan(out), torch.isnan(ref))
+    assert torch.equal(torch.isposinf(out), torch.isposinf(ref)) and torch.equal(torch.isneginf(out), torch.isneginf(ref))
+    fin = torch.isfinite(ref)
+    assert ((out[fin] - ref[fin]).abs().max() / ref[fin].abs().max()).item() < 2e-4
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 384, 512), (300, 520, 200), (16, 1024, 4096), (1000, 72, 1003)])

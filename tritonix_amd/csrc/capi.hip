@@ -502,17 +502,21 @@ __global__ void split_f32_kernel(const float* src, int64_t rows, int64_t cols, i
   const float v = src[i * sr + j * sc];
   const __bf16 hi = (__bf16)v;                                        // round to nearest even
   const float rest = v - (float)hi;
-  const __bf16 lo = (__builtin_isfinite(rest) && __builtin_isfinite(v)) ? (__bf16)rest : (__bf16)0.0f;
+  // An infinity or NaN lives in the head alone: its tail is zero, and so is the second copy of its head -- the one
+  // that meets the other operand's tail -- or inf * (a tail that happens to be 0) would turn an infinite sum into NaN.
+  const bool fin = __builtin_isfinite(rest) && __builtin_isfinite((float)hi);
+  const __bf16 lo = fin ? (__bf16)rest : (__bf16)0.0f;
   const uint16_t h = __builtin_bit_cast(uint16_t, hi), l = __builtin_bit_cast(uint16_t, lo);
+  const uint16_t h2 = fin ? h : (uint16_t)0;
   if (side == 0 || side == 2) {
     uint16_t* row = dst + i * 3 * cols;
     row[j] = h;
-    row[cols + j] = side == 0 ? h : l;
-    row[2 * cols + j] = side == 0 ? l : h;
+    row[cols + j] = side == 0 ? h2 : l;
+    row[2 * cols + j] = side == 0 ? l : h2;
   } else {
     dst[i * cols + j] = h;
     dst[(rows + i) * cols + j] = l;
-    dst[(2 * rows + i) * cols + j] = h;
+    dst[(2 * rows + i) * cols + j] = h2;
   }
 }
 
